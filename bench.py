@@ -1,0 +1,220 @@
+"""Benchmark of the scattered-MoE layer forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+A step is one forward of the MoE layer (router -> sort/bin -> up-projection + SwiGLU -> down-projection
+-> combine) over one batch of seeded synthetic tokens that already sit in HBM.  The default workload is
+the Granite-3B-A800M-shape layer (32768 tokens, hidden 1536, 40 experts, top-8, intermediate 512, bf16,
+Zipf(1.1) expert load).  One JSON line is printed:
+
+* ``value``         tokens/s of the whole forward, K steps between two device synchronisations
+* ``roofline``      the dominant kernel (grouped up-projection GEMM with fused SwiGLU; for the decode
+                    workload the fp8 up-projection weight stream): algorithmic flops (or bytes) per
+                    launch / average launch duration, measured with HIP events on the launch stream
+                    in a second, instrumented run of the same K steps
+* ``cpu_baseline``  the eager per-expert-loop path (the oracle, a port of the reference's eager
+                    branch) in fp32 on the host cores, on a bounded token sample of the same workload
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+class StageTimer:
+    """HIP events (torch.cuda.Event on the current stream, which is the stream the kernels are
+    launched on) around every stage of the forward."""
+
+    def __init__(self):
+        import torch
+
+        self.torch = torch
+        self.events = {}
+        self._open = {}
+
+    def begin(self, name):
+        ev = self.torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self._open[name] = ev
+
+    def end(self, name):
+        ev = self.torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.events.setdefault(name, []).append((self._open.pop(name), ev))
+
+    def summary(self):
+        self.torch.cuda.synchronize()
+        return {n: sum(a.elapsed_time(b) for a, b in evs) / len(evs) for n, evs in self.events.items()}
+
+
+def build_module(w, inputs, device):
+    import torch
+
+    from dolomite_engine_amd import MoE
+
+    with torch.device("meta"):
+        m = MoE(hidden_size=w.H, intermediate_size=w.I, shared_intermediate_size=None, num_experts=w.E,
+                num_experts_per_tok=w.k, activation_function="swiglu", add_bias=False, dropout=0.0,
+                init_method="normal", initializer_range=0.02, m_width=None, num_layers=1,
+                use_padding_free_transformer=True)
+    m = m.to(w.dtype).to_empty(device=device).eval()
+    with torch.no_grad():
+        m.gate.weight.copy_(inputs["gate_w"])
+        if w.fp8:
+            m.c_fc.weight = None
+            m.c_proj.weight = None
+            m.c_fc.weight_q = inputs["w_fc"].to(device)
+            m.c_fc.weight_scale = inputs["fc_scale"].to(device)
+            m.c_proj.weight_q = inputs["w_proj"].to(device)
+            m.c_proj.weight_scale = inputs["proj_scale"].to(device)
+            m.c_fc.weight_scale_dtype = m.c_proj.weight_scale_dtype = w.dtype
+        else:
+            m.c_fc.weight.copy_(inputs["w_fc"])
+            m.c_proj.weight.copy_(inputs["w_proj"])
+    if inputs["bias"] is not None:
+        m.router_logit_bias = inputs["bias"].to(device)
+    return m
+
+
+def cpu_baseline(w, inputs, sample_tokens, iters=3):
+    """Eager path of the oracle in fp32 on the host, on the first ``sample_tokens`` tokens."""
+    import torch
+
+    from oracle import moe_oracle as oracle
+
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    x = inputs["x"][:sample_tokens].float()
+    gate_w = inputs["gate_w"].float()
+    if w.fp8:
+        w_fc = oracle.dequant_fp8(inputs["w_fc"], inputs["fc_scale"])
+        w_proj = oracle.dequant_fp8(inputs["w_proj"], inputs["proj_scale"])
+    else:
+        w_fc, w_proj = inputs["w_fc"].float(), inputs["w_proj"].float()
+    bias = inputs["bias"]
+
+    def run():
+        _, gates, idx = oracle.route(x, gate_w, w.k, bias=bias)
+        return oracle.experts_eager(x, gates, idx, w_fc, w_proj)
+
+    run()
+    times = []
+    for _ in range(iters):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {
+        "value": sample_tokens / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"first {sample_tokens} tokens of the workload, fp32 eager per-expert loop, 1 warm-up + {iters} "
+                  f"timed forwards, median {med * 1e3:.1f} ms; host has {os.cpu_count()} logical cpus",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="granite-3b-a800m")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=None)
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (one GPU's share of the layer at its real shape); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from dolomite_engine_amd import Kernel, enable_kernels, ops
+    from oracle import moe_oracle as oracle
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    w = oracle.WORKLOADS[args.workload]
+    inputs = oracle.make_inputs(w)
+    m = build_module(w, inputs, device)
+    x = inputs["x"].to(device)
+    T, H, E, k, I = w.T, w.H, w.E, w.k, w.I
+    L = T * k
+
+    with torch.no_grad(), enable_kernels([Kernel.scattermoe]):
+        for _ in range(args.warmup):
+            y = m(x)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            y = m(x)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+
+        # instrumented run of the same steps: HIP events around every stage
+        timer = StageTimer()
+        ops.set_stage_timer(timer)
+        for _ in range(args.steps):
+            y = m(x)
+        stages = timer.summary()
+        ops.set_stage_timer(None)
+
+        idx = ops.router_fused(x, m.gate.weight, k, bias=m.router_logit_bias)[2]
+        counts = torch.bincount(idx.flatten().long(), minlength=E).cpu()
+
+    ms_per_step = elapsed / args.steps * 1e3
+    tokens_per_s = T / (elapsed / args.steps)
+    flops = 6.0 * L * H * I
+    touched = int((counts > 0).sum())
+
+    if w.fp8:
+        up_name = "up_swiglu_fp8"
+        up_bytes = touched * (2 * I * H) + touched * 2 * I * 4 + T * H * 2 + L * I * 2 + L * 4 + E * 4
+        ach = up_bytes / (stages[up_name] * 1e-3) / 1e9
+        roofline = {"kernel": up_name, "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": ach / PEAK_HBM_GBS, "traffic": None, "algorithmic_bytes": up_bytes,
+                    "avg_launch_ms": stages[up_name]}
+    else:
+        up_name = "up_swiglu"
+        up_flops = 4.0 * L * H * I
+        ach = up_flops / (stages[up_name] * 1e-3) / 1e12
+        roofline = {"kernel": up_name, "bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS,
+                    "unit": "TFLOP/s", "frac": ach / PEAK_BF16_TFLOPS, "traffic": None,
+                    "algorithmic_flops": up_flops, "avg_launch_ms": stages[up_name]}
+        if "scattered_gemm" in stages:
+            down = 2.0 * L * H * I / (stages["scattered_gemm"] * 1e-3) / 1e12
+            roofline["down_gemm_tflops"] = down
+            roofline["both_gemms_frac"] = flops / ((stages[up_name] + stages["scattered_gemm"]) * 1e-3) / 1e12 / PEAK_BF16_TFLOPS
+
+    out = {
+        "metric": "MoE fwd tokens/s & % bf16 MFMA peak, Granite-3B-A800M layer, 1 GPU",
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if not w.fp8 else "bf16 activations, fp8-e4m3 weights", "data": "synthetic",
+        "config": {"workload": w.name, "tokens": T, "hidden": H, "experts": E, "top_k": k, "intermediate": I,
+                   "expert_load": "zipf(1.1) first-choice" if w.zipf_s else "near-uniform",
+                   "experts_touched": touched, "max_over_min_load": float(counts.max()) / max(1.0, float(counts.min()))},
+        "layer_tflops": flops / (elapsed / args.steps) / 1e12,
+        "stages_ms": stages,
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        sample = args.cpu_sample_tokens or min(T, 8192)
+        out["cpu_baseline"] = cpu_baseline(w, inputs, sample)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

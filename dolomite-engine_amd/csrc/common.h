@@ -1,0 +1,88 @@
+// Shared device/host helpers for the gfx950 scattered-MoE kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mi_moe.h"
+
+#define MI_WAVE 64
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// ---- element conversions (round-to-nearest-even, like torch's casts) -------------------------
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T> struct Elt;
+template <> struct Elt<float> {
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+template <> struct Elt<bf16_t> {
+  static __device__ __forceinline__ float load(const bf16_t* p) {
+    return bf16_bits_to_float(*reinterpret_cast<const uint16_t*>(p));
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, float v) {
+    *reinterpret_cast<uint16_t*>(p) = float_to_bf16_bits(v);
+  }
+  static __device__ __forceinline__ float round(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
+};
+template <> struct Elt<f16_t> {
+  static __device__ __forceinline__ float load(const f16_t* p) { return (float)(*p); }
+  static __device__ __forceinline__ void store(f16_t* p, float v) { *p = (f16_t)v; }
+  static __device__ __forceinline__ float round(float v) { return (float)((f16_t)v); }
+};
+
+// pack two floats into two 16-bit elements of type T (low half = a)
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
+  return (uint32_t)float_to_bf16_bits(a) | ((uint32_t)float_to_bf16_bits(b) << 16);
+}
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
+  f16_t ha = (f16_t)a, hb = (f16_t)b;
+  return (uint32_t)(*reinterpret_cast<uint16_t*>(&ha)) | ((uint32_t)(*reinterpret_cast<uint16_t*>(&hb)) << 16);
+}
+
+template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t v);
+template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t v);
+template <> __device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t v) { return __uint_as_float(v << 16); }
+template <> __device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t v) { return __uint_as_float(v & 0xffff0000u); }
+template <> __device__ __forceinline__ float unpack_lo<f16_t>(uint32_t v) {
+  uint16_t h = (uint16_t)(v & 0xffffu);
+  return (float)(*reinterpret_cast<f16_t*>(&h));
+}
+template <> __device__ __forceinline__ float unpack_hi<f16_t>(uint32_t v) {
+  uint16_t h = (uint16_t)(v >> 16);
+  return (float)(*reinterpret_cast<f16_t*>(&h));
+}
+
+__device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
+
+// ---- host helpers ---------------------------------------------------------------------------
+
+static inline int mi_launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? MI_MOE_OK : (int)e;
+}
+
+static inline bool mi_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+static inline int mi_ceil_div(int a, int b) { return (a + b - 1) / b; }
+__device__ __forceinline__ int mi_ceil_div_dev(int a, int b) { return (a + b - 1) / b; }

@@ -1,0 +1,215 @@
+// Decode-shape (few rows per expert) grouped GEMM with fp8 e4m3fn expert weights and one fp32 scale
+// per output channel:   out[orow(i), n] = scale[e_i, n] * sum_k in[irow(i), k] * Wq[e_i, n, k]
+// optionally with the SwiGLU epilogue (weight rows [0,N) "up", [N,2N) "gate").
+//
+// The reference has no fp8 expert path (lm_engine/fp8.py:63-73 converts nn.Linear only); the
+// semantics are "dequantise, then lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:273-290".
+//
+// The shape is weight-streaming bound: with ~6 rows per expert every weight byte is used once, so
+// the kernel is organised around the weight stream.
+//   * grid = experts x column-tile groups; an expert with no rows exits at once, so only the weights
+//     of touched experts are read, each exactly once (row groups beyond 16 re-read from L2).
+//   * a wavefront owns 16 output channels (x2 for SwiGLU): lane (r = l%16, q = l/16) streams weight
+//     row r, 16 consecutive fp8 per load (one dwordx4), i.e. each 64-wide K step is one fully used
+//     128-byte line per weight row.  The bytes are widened to bf16/f16 in registers (exact) and used as
+//     the A operand of v_mfma_f32_16x16x32; the B operand is the matching 16-row activation slice.
+//     A and B use the same lane->k assignment, so no shuffle is needed to match the MFMA's own k order.
+//   * KSPLIT wavefronts of a workgroup share one column tile and split K between them (more loads in
+//     flight per weight row); partial sums meet in LDS.
+//   * the per-channel scale, SwiGLU and the 8-byte packed store happen in the epilogue.
+#include "common.h"
+
+template <typename T> struct Mfma16;
+template <> struct Mfma16<bf16_t> {
+  typedef bf16x8 vec;
+  static __device__ __forceinline__ f32x4 run(vec a, vec b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  // 8 fp8 (two dwords) -> 8 bf16; exact, e4m3 fits in bf16
+  static __device__ __forceinline__ vec widen(uint32_t lo, uint32_t hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
+    bf16x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+    bf16x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
+    bf16x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+    vec v = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+    return v;
+  }
+};
+template <> struct Mfma16<f16_t> {
+  typedef f16x8 vec;
+  static __device__ __forceinline__ f32x4 run(vec a, vec b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ vec widen(uint32_t lo, uint32_t hi) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false);
+    f32x2 p1 = __builtin_amdgcn_cvt_pk_f32_fp8(lo, true);
+    f32x2 p2 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
+    f32x2 p3 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+    vec v = {(f16_t)p0[0], (f16_t)p0[1], (f16_t)p1[0], (f16_t)p1[1],
+             (f16_t)p2[0], (f16_t)p2[1], (f16_t)p3[0], (f16_t)p3[1]};
+    return v;
+  }
+};
+
+struct DecodeArgs {
+  const void* in;
+  const uint8_t* wq;
+  const float* scale;
+  void* out;
+  const int32_t* sorted_scattered;
+  const int32_t* expert_offsets;
+  int L, K, N, E, kdiv;
+  int gather, scatter;
+  int groups_per_expert;  // workgroups per expert
+};
+
+template <typename T, bool GLU, int KSPLIT>
+__global__ __launch_bounds__(256) void decode_fp8_kernel(DecodeArgs a) {
+  constexpr int NTB = 4 / KSPLIT;  // 16-channel column tiles per workgroup
+  constexpr int WR = GLU ? 2 : 1;
+  typedef typename Mfma16<T>::vec frag_t;
+  __shared__ f32x4 red[4][2][64];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int expert = blockIdx.x / a.groups_per_expert;
+  const int grp = blockIdx.x - expert * a.groups_per_expert;
+  const int row_begin = expert ? a.expert_offsets[expert - 1] : 0;
+  const int row_end = a.expert_offsets[expert];
+  if (row_begin >= row_end) return;  // whole workgroup: nothing routed here, weights stay untouched
+
+  const int ks = wave % KSPLIT;
+  const int n0 = (grp * NTB + wave / KSPLIT) * 16;
+  int wrow = n0 + r;
+  if (wrow > a.N - 1) wrow = a.N - 1;  // column tail re-reads the last channel; never stored
+  const uint8_t* __restrict__ wu = a.wq + ((size_t)expert * WR * a.N + wrow) * a.K;
+  const uint8_t* __restrict__ wg = wu + (size_t)a.N * a.K;
+
+  const int ksteps = (a.K + 63) >> 6;
+  const int per = (ksteps + KSPLIT - 1) / KSPLIT;
+  const int s_begin = ks * per;
+  int s_end = s_begin + per;
+  if (s_end > ksteps) s_end = ksteps;
+
+  const T* __restrict__ xin = static_cast<const T*>(a.in);
+  T* __restrict__ out = static_cast<T*>(a.out);
+
+  for (int g0 = row_begin; g0 < row_end; g0 += 16) {
+    int srow = g0 + r;
+    if (srow > row_end - 1) srow = row_end - 1;  // short group re-reads the last row; never stored
+    const int slot = (a.gather || a.scatter) ? a.sorted_scattered[srow] : 0;
+    const int src = a.gather ? slot / a.kdiv : srow;
+    const T* __restrict__ xp = xin + (size_t)src * a.K;
+
+    f32x4 acc_u = {0.f, 0.f, 0.f, 0.f}, acc_g = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int s = s_begin; s < s_end; ++s) {
+      const int kpos = s * 64 + q * 16;
+      u32x4 wub = {0u, 0u, 0u, 0u}, wgb = {0u, 0u, 0u, 0u}, x0 = {0u, 0u, 0u, 0u}, x1 = {0u, 0u, 0u, 0u};
+      if (kpos < a.K) {
+        wub = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wu + kpos));
+        if (GLU) wgb = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wg + kpos));
+        x0 = *reinterpret_cast<const u32x4*>(xp + kpos);
+        x1 = *reinterpret_cast<const u32x4*>(xp + kpos + 8);
+      }
+      const frag_t b0 = __builtin_bit_cast(frag_t, x0), b1 = __builtin_bit_cast(frag_t, x1);
+      acc_u = Mfma16<T>::run(Mfma16<T>::widen(wub[0], wub[1]), b0, acc_u);
+      acc_u = Mfma16<T>::run(Mfma16<T>::widen(wub[2], wub[3]), b1, acc_u);
+      if (GLU) {
+        acc_g = Mfma16<T>::run(Mfma16<T>::widen(wgb[0], wgb[1]), b0, acc_g);
+        acc_g = Mfma16<T>::run(Mfma16<T>::widen(wgb[2], wgb[3]), b1, acc_g);
+      }
+    }
+
+    if (KSPLIT > 1) {
+      if (ks != 0) {
+        red[wave][0][lane] = acc_u;
+        if (GLU) red[wave][1][lane] = acc_g;
+      }
+      __syncthreads();
+      if (ks == 0) {
+#pragma unroll
+        for (int o = 1; o < KSPLIT; ++o) {
+          f32x4 pu = red[wave + o][0][lane];
+          acc_u += pu;
+          if (GLU) {
+            f32x4 pg = red[wave + o][1][lane];
+            acc_g += pg;
+          }
+        }
+      }
+      __syncthreads();
+    }
+
+    // acc[i]: output channel n0 + 4q + i, row g0 + r
+    const int col = n0 + 4 * q;
+    if (ks == 0 && g0 + r < row_end && col < a.N) {
+      const float* su = a.scale + (size_t)expert * WR * a.N + col;
+      const f32x4 scu = *reinterpret_cast<const f32x4*>(su);
+      float v[4];
+      if (GLU) {
+        const f32x4 scg = *reinterpret_cast<const f32x4*>(su + a.N);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = (acc_u[i] * scu[i]) * silu_f32(acc_g[i] * scg[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = acc_u[i] * scu[i];
+      }
+      const int orow = a.scatter ? slot : g0 + r;
+      u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+      *reinterpret_cast<u32x2*>(out + (size_t)orow * a.N + col) = p;
+    }
+  }
+}
+
+template <typename T, bool GLU, int KSPLIT>
+static int launch_decode(DecodeArgs a, hipStream_t s) {
+  constexpr int NTB = 4 / KSPLIT;
+  a.groups_per_expert = mi_ceil_div(a.N, 16 * NTB);
+  long grid = (long)a.E * a.groups_per_expert;
+  if (grid > 0x7fffffffL) return MI_MOE_ESHAPE;
+  hipLaunchKernelGGL((decode_fp8_kernel<T, GLU, KSPLIT>), dim3((unsigned)grid), dim3(256), 0, s, a);
+  return mi_launch_status();
+}
+
+template <typename T, bool GLU>
+static int dispatch_decode(const DecodeArgs& a, hipStream_t s) {
+  if (a.K >= 2048) return launch_decode<T, GLU, 4>(a, s);
+  if (a.K >= 1024) return launch_decode<T, GLU, 2>(a, s);
+  return launch_decode<T, GLU, 1>(a, s);
+}
+
+static int run_decode(DecodeArgs a, int dtype, bool glu, hipStream_t s) {
+  if (a.L < 0 || a.K < 1 || a.N < 1 || a.E < 1 || a.kdiv < 1) return MI_MOE_ESHAPE;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (a.L == 0) return MI_MOE_OK;
+  if (!a.in || !a.wq || !a.scale || !a.out || !a.expert_offsets) return MI_MOE_ENULL;
+  if ((a.gather || a.scatter) && !a.sorted_scattered) return MI_MOE_ENULL;
+  if (a.K % 16 != 0 || a.N % 4 != 0) return MI_MOE_EUNSUPPORTED;
+  if (!mi_aligned(a.in, 16) || !mi_aligned(a.wq, 16) || !mi_aligned(a.scale, 16) || !mi_aligned(a.out, 8))
+    return MI_MOE_EALIGN;
+  if (dtype == MI_MOE_BF16) return glu ? dispatch_decode<bf16_t, true>(a, s) : dispatch_decode<bf16_t, false>(a, s);
+  return glu ? dispatch_decode<f16_t, true>(a, s) : dispatch_decode<f16_t, false>(a, s);
+}
+
+extern "C" int mi_moe_up_swiglu_fp8(const void* x, const void* w_fc_q, const float* w_fc_scale, void* act_out,
+                                    const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int H,
+                                    int I, int E, int k, int dtype, mi_moe_stream_t stream) {
+  DecodeArgs a;
+  a.in = x; a.wq = static_cast<const uint8_t*>(w_fc_q); a.scale = w_fc_scale; a.out = act_out;
+  a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
+  a.L = L; a.K = H; a.N = I; a.E = E; a.kdiv = k; a.gather = 1; a.scatter = 0; a.groups_per_expert = 0;
+  return run_decode(a, dtype, true, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mi_moe_down_fp8(const void* act, const void* w_proj_q, const float* w_proj_scale, void* o_out,
+                               const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
+                               int E, int dtype, mi_moe_stream_t stream) {
+  DecodeArgs a;
+  a.in = act; a.wq = static_cast<const uint8_t*>(w_proj_q); a.scale = w_proj_scale; a.out = o_out;
+  a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
+  a.L = L; a.K = I; a.N = H; a.E = E; a.kdiv = 1; a.gather = 0; a.scatter = 1; a.groups_per_expert = 0;
+  return run_decode(a, dtype, false, static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,196 @@
+// Fused router: logits = x @ gate_w^T (rounded to the model dtype, optional bias), top-k with the
+// canonical tie rule, fp32 softmax over the k winners -- one pass over x, nothing but the (T,k)
+// results (and optionally the logits) written.
+// Stands in for MoE._compute_routing_weights, lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:246-257.
+//
+// HBM-bound on reading x.  A wavefront owns TG groups of 16 tokens and all (<= 64) experts:
+//   * v_mfma_f32_16x16x32 with the gate weights as operand A (16 experts x 32 k) and the tokens as
+//     operand B, so lane (r = l%16, q = l/16) ends with logits of token r for experts 16*eb + 4q + i;
+//   * lane (r, q) streams 16 consecutive k of its token row per 64-wide K step (two dwordx4), so the four
+//     q-lanes of a token cover one full 128-byte line; both operands use that same lane->k assignment;
+//   * top-k: a token's 64 candidates live in 4 lanes x 16 registers; each of the k rounds takes a
+//     per-lane maximum of 64-bit keys (ordered value << 32 | ~expert) and a 2-step butterfly.
+#include "common.h"
+
+template <typename T> struct RMfma;
+template <> struct RMfma<bf16_t> {
+  typedef bf16x8 vec;
+  static __device__ __forceinline__ f32x4 run(vec a, vec b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct RMfma<f16_t> {
+  typedef f16x8 vec;
+  static __device__ __forceinline__ f32x4 run(vec a, vec b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+__device__ __forceinline__ uint32_t router_ordered_key(float v) {
+  uint32_t u = __float_as_uint(v);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;
+  if (u == 0x80000000u) u = 0u;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+#define ROUTER_KMAX 8
+
+template <typename T, int TG>
+__global__ __launch_bounds__(256) void router_fused_kernel(const T* __restrict__ x, const T* __restrict__ gw,
+                                                           const float* __restrict__ bias, int Trows, int H, int E,
+                                                           int k, T* __restrict__ logits_out, T* __restrict__ gates,
+                                                           int32_t* __restrict__ idx) {
+  typedef typename RMfma<T>::vec frag_t;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int tok0 = (blockIdx.x * 4 + wave) * (16 * TG);
+  if (tok0 >= Trows) return;
+
+  const T* xrow[TG];
+#pragma unroll
+  for (int g = 0; g < TG; ++g) {
+    int t = tok0 + g * 16 + r;
+    if (t > Trows - 1) t = Trows - 1;
+    xrow[g] = x + (size_t)t * H;
+  }
+  const T* wrow[4];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) {
+    int e = eb * 16 + r;
+    if (e > E - 1) e = E - 1;
+    wrow[eb] = gw + (size_t)e * H;
+  }
+
+  f32x4 acc[4][TG];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb)
+#pragma unroll
+    for (int g = 0; g < TG; ++g) acc[eb][g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll 2
+  for (int k0 = 0; k0 < H; k0 += 64) {
+    const int kpos = k0 + q * 16;
+    const bool valid = kpos < H;
+    u32x4 xa[TG][2], wa[4][2];
+#pragma unroll
+    for (int g = 0; g < TG; ++g) {
+      xa[g][0] = xa[g][1] = (u32x4){0u, 0u, 0u, 0u};
+      if (valid) {
+        xa[g][0] = *reinterpret_cast<const u32x4*>(xrow[g] + kpos);
+        xa[g][1] = *reinterpret_cast<const u32x4*>(xrow[g] + kpos + 8);
+      }
+    }
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) {
+      wa[eb][0] = wa[eb][1] = (u32x4){0u, 0u, 0u, 0u};
+      if (valid) {
+        wa[eb][0] = *reinterpret_cast<const u32x4*>(wrow[eb] + kpos);
+        wa[eb][1] = *reinterpret_cast<const u32x4*>(wrow[eb] + kpos + 8);
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int eb = 0; eb < 4; ++eb)
+#pragma unroll
+        for (int g = 0; g < TG; ++g)
+          acc[eb][g] = RMfma<T>::run(__builtin_bit_cast(frag_t, wa[eb][h]), __builtin_bit_cast(frag_t, xa[g][h]),
+                                     acc[eb][g]);
+  }
+
+  // ---- epilogue: round, bias, optional logits store, top-k, softmax ---------------------------
+#pragma unroll
+  for (int g = 0; g < TG; ++g) {
+    const int t = tok0 + g * 16 + r;
+    const bool tvalid = t < Trows;
+    uint64_t keys[16];
+    float vals[16];
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int e = eb * 16 + 4 * q + i;
+        float v = Elt<T>::round(acc[eb][g][i]);
+        if (bias != nullptr && e < E) v = Elt<T>::round(v + bias[e]);
+        vals[eb * 4 + i] = v;
+        keys[eb * 4 + i] = e < E ? (((uint64_t)router_ordered_key(v) << 32) | (uint32_t)(~(uint32_t)e)) : 0ull;
+        if (logits_out != nullptr && tvalid && e < E) Elt<T>::store(logits_out + (size_t)t * E + e, v);
+      }
+    }
+    float wv[ROUTER_KMAX];
+    int wi[ROUTER_KMAX];
+#pragma unroll
+    for (int j = 0; j < ROUTER_KMAX; ++j) {
+      wv[j] = 0.f;
+      wi[j] = 0;
+      if (j < k) {
+        uint64_t best = 0ull;
+        float bv = 0.f;
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+          if (keys[c] > best) {
+            best = keys[c];
+            bv = vals[c];
+          }
+        }
+#pragma unroll
+        for (int off = 16; off <= 32; off <<= 1) {
+          uint32_t lo = __shfl_xor((uint32_t)best, off, MI_WAVE);
+          uint32_t hi = __shfl_xor((uint32_t)(best >> 32), off, MI_WAVE);
+          float ov = __shfl_xor(bv, off, MI_WAVE);
+          uint64_t o = ((uint64_t)hi << 32) | lo;
+          if (o > best) {
+            best = o;
+            bv = ov;
+          }
+        }
+#pragma unroll
+        for (int c = 0; c < 16; ++c)
+          if (keys[c] == best) keys[c] = 0ull;
+        wv[j] = bv;
+        wi[j] = (int)(~(uint32_t)best);
+      }
+    }
+    if (q == 0 && tvalid) {
+      float p[ROUTER_KMAX];
+      float denom = 0.f;
+#pragma unroll
+      for (int j = 0; j < ROUTER_KMAX; ++j) {
+        p[j] = j < k ? expf(wv[j] - wv[0]) : 0.f;
+        denom += p[j];
+      }
+#pragma unroll
+      for (int j = 0; j < ROUTER_KMAX; ++j) {
+        if (j < k) {
+          Elt<T>::store(gates + (size_t)t * k + j, p[j] / denom);
+          idx[(size_t)t * k + j] = wi[j];
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+static int launch_router(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
+                         void* logits_out, void* gates, int32_t* idx, hipStream_t s) {
+  constexpr int TG = 2;
+  dim3 grid(mi_ceil_div(T_, 4 * 16 * TG)), block(256);
+  hipLaunchKernelGGL((router_fused_kernel<T, TG>), grid, block, 0, s, static_cast<const T*>(x),
+                     static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out),
+                     static_cast<T*>(gates), idx);
+  return mi_launch_status();
+}
+
+extern "C" int mi_moe_router_fused(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,
+                                   int dtype, void* logits_out, void* gates_out, int32_t* idx_out,
+                                   mi_moe_stream_t stream) {
+  if (T < 0 || H < 1 || E < 1 || k < 1 || k > E) return MI_MOE_ESHAPE;
+  if (E > 64 || k > ROUTER_KMAX || H % 16 != 0) return MI_MOE_EUNSUPPORTED;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (T == 0) return MI_MOE_OK;
+  if (!x || !gate_w || !gates_out || !idx_out) return MI_MOE_ENULL;
+  if (!mi_aligned(x, 16) || !mi_aligned(gate_w, 16)) return MI_MOE_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MI_MOE_BF16) return launch_router<bf16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, s);
+  return launch_router<f16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, s);
+}

@@ -1,0 +1,407 @@
+// Routing stage of the scattered-MoE forward on gfx950:
+//   * top-k + softmax over the selected logits (wave64 shuffle reductions, one row per wavefront)
+//   * expert histogram
+//   * stable counting sort of the flat expert ids (LDS histograms -> prefix sums -> stable scatter)
+//
+// Stands in for lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:250-255, 263-271, 338-344 and
+// the external continuous_count op used at moe.py:38-44.
+#include "common.h"
+
+// ------------------------------------------------------------------------------------------------
+// top-k softmax
+// ------------------------------------------------------------------------------------------------
+
+// Order-preserving map float -> uint32 (larger float <=> larger key); NaN is the largest key and
+// -0.0 is folded onto +0.0 so that it ties with it, as a floating-point comparison would.
+__device__ __forceinline__ uint32_t ordered_key(float v) {
+  uint32_t u = __float_as_uint(v);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;
+  if (u == 0x80000000u) u = 0u;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    uint32_t lo = __shfl_xor((uint32_t)v, off, MI_WAVE);
+    uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, MI_WAVE);
+    uint64_t o = ((uint64_t)hi << 32) | lo;
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, MI_WAVE);
+  return v;
+}
+
+// One wavefront per row.  Lane l owns experts l, l+64, ... (VPL of them).  A candidate is the
+// 64-bit key (ordered(value) << 32) | ~expert, so a plain unsigned max implements "value
+// descending, expert index ascending".  Round j finds the j-th winner with a butterfly max; the
+// lane that owns it retires it.  Lane j keeps winner j, then lanes [0,k) do the softmax.
+template <typename T, int VPL>
+__global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__ logits, int Trows, int E, int k,
+                                                           T* __restrict__ gates, int32_t* __restrict__ idx) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= Trows) return;
+  const T* src = logits + (size_t)row * E;
+
+  float vals[VPL];
+  uint64_t keys[VPL];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    int e = lane + i * 64;
+    if (e < E) {
+      vals[i] = Elt<T>::load(src + e);
+      keys[i] = ((uint64_t)ordered_key(vals[i]) << 32) | (uint32_t)(~(uint32_t)e);
+    } else {
+      vals[i] = 0.f;
+      keys[i] = 0ull;  // below every real candidate (real keys have a non-zero low word)
+    }
+  }
+
+  float my_val = 0.f;
+  int my_idx = 0;
+  for (int j = 0; j < k; ++j) {
+    uint64_t best = 0ull;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) best = keys[i] > best ? keys[i] : best;
+    best = wave_max_u64(best);
+    int e = (int)(~(uint32_t)best);
+    // the owner retires the winner and publishes its value
+    float v = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      if (keys[i] == best) {
+        v = vals[i];
+        keys[i] = 0ull;
+      }
+    }
+    v = __shfl(v, e & 63, MI_WAVE);
+    if (lane == j) {
+      my_val = v;
+      my_idx = e;
+    }
+  }
+
+  // softmax over the k winners in fp32; winner 0 is the maximum
+  float vmax = __shfl(my_val, 0, MI_WAVE);
+  float p = (lane < k) ? expf(my_val - vmax) : 0.f;
+  float denom = wave_sum_f32(p);
+  if (lane < k) {
+    Elt<T>::store(gates + (size_t)row * k + lane, p / denom);
+    idx[(size_t)row * k + lane] = my_idx;
+  }
+}
+
+template <typename T>
+static int launch_topk(const void* logits, int T_, int E, int k, void* gates, int32_t* idx, hipStream_t s) {
+  dim3 grid(mi_ceil_div(T_, 4)), block(256);
+  const T* lg = static_cast<const T*>(logits);
+  T* gt = static_cast<T*>(gates);
+  if (E <= 64)
+    hipLaunchKernelGGL((topk_softmax_kernel<T, 1>), grid, block, 0, s, lg, T_, E, k, gt, idx);
+  else if (E <= 128)
+    hipLaunchKernelGGL((topk_softmax_kernel<T, 2>), grid, block, 0, s, lg, T_, E, k, gt, idx);
+  else if (E <= 256)
+    hipLaunchKernelGGL((topk_softmax_kernel<T, 4>), grid, block, 0, s, lg, T_, E, k, gt, idx);
+  else
+    hipLaunchKernelGGL((topk_softmax_kernel<T, 16>), grid, block, 0, s, lg, T_, E, k, gt, idx);
+  return mi_launch_status();
+}
+
+extern "C" int mi_moe_router_topk_softmax(const void* logits, int T, int E, int k, int dtype, void* gates_out,
+                                          int32_t* idx_out, mi_moe_stream_t stream) {
+  if (T < 0 || E < 1 || E > 1024 || k < 1 || k > E || k > 64) return MI_MOE_ESHAPE;
+  if (T == 0) return MI_MOE_OK;
+  if (!logits || !gates_out || !idx_out) return MI_MOE_ENULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case MI_MOE_F32: return launch_topk<float>(logits, T, E, k, gates_out, idx_out, s);
+    case MI_MOE_F16: return launch_topk<f16_t>(logits, T, E, k, gates_out, idx_out, s);
+    case MI_MOE_BF16: return launch_topk<bf16_t>(logits, T, E, k, gates_out, idx_out, s);
+    default: return MI_MOE_EDTYPE;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// histogram of expert ids
+// ------------------------------------------------------------------------------------------------
+
+__global__ void zero_u32_kernel(uint32_t* p, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+__global__ __launch_bounds__(256) void count_kernel(const int32_t* __restrict__ ids, int L, int E,
+                                                    uint32_t* __restrict__ counts) {
+  __shared__ uint32_t hist[1024];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) hist[e] = 0u;
+  __syncthreads();
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < L; i += gridDim.x * blockDim.x) {
+    int e = ids[i];
+    if ((unsigned)e < (unsigned)E) atomicAdd(&hist[e], 1u);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    uint32_t c = hist[e];
+    if (c) atomicAdd(&counts[e], c);
+  }
+}
+
+extern "C" int mi_moe_count(const int32_t* ids, int L, int E, uint32_t* counts_out, mi_moe_stream_t stream) {
+  if (L < 0 || E < 1 || E > 1024) return MI_MOE_ESHAPE;
+  if (!counts_out || (L > 0 && !ids)) return MI_MOE_ENULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(zero_u32_kernel, dim3(mi_ceil_div(E, 256)), dim3(256), 0, s, counts_out, E);
+  if (L > 0) {
+    int blocks = mi_ceil_div(L, 256 * 8);
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(count_kernel, dim3(blocks), dim3(256), 0, s, ids, L, E, counts_out);
+  }
+  return mi_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// stable counting sort of expert ids
+// ------------------------------------------------------------------------------------------------
+//
+// The L slots are cut into chunks of SORT_CHUNK consecutive slots, one block per chunk.
+//   pass 1  per-chunk histogram in LDS                   -> ws[e * nblk + b]
+//   pass 2  per expert: exclusive scan over the chunks (in place); scan over the experts gives the
+//           inclusive expert_offsets (output) and the exclusive expert bases (ws tail)
+//   pass 3  each chunk is re-read in order; wave w of the block owns a contiguous quarter of the
+//           chunk and walks it 64 slots at a time, so "earlier slot" == "earlier wave, earlier step,
+//           lower lane" and ranks come from a match-any ballot: the scatter is stable.
+// Small inputs (one chunk) run all three passes inside a single block and need no workspace.
+
+#define SORT_THREADS 256
+#define SORT_WAVES (SORT_THREADS / 64)
+#define SORT_CHUNK 2048
+#define SORT_MAX_E 1024
+
+__global__ __launch_bounds__(SORT_THREADS) void sort_hist_kernel(const int32_t* __restrict__ ids, int L, int E,
+                                                                 int nblk, int32_t* __restrict__ ws) {
+  __shared__ int hist[SORT_MAX_E];
+  for (int e = threadIdx.x; e < E; e += SORT_THREADS) hist[e] = 0;
+  __syncthreads();
+  const int base = blockIdx.x * SORT_CHUNK;
+#pragma unroll
+  for (int j = 0; j < SORT_CHUNK / SORT_THREADS; ++j) {
+    int i = base + j * SORT_THREADS + threadIdx.x;
+    if (i < L) {
+      int e = ids[i];
+      if ((unsigned)e < (unsigned)E) atomicAdd(&hist[e], 1);
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += SORT_THREADS) ws[(size_t)e * nblk + blockIdx.x] = hist[e];
+}
+
+__device__ __forceinline__ int wave_incl_scan_i32(int v, int lane) {
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    int o = __shfl_up(v, off, MI_WAVE);
+    if (lane >= off) v += o;
+  }
+  return v;
+}
+
+// single block of 1024 threads (16 waves)
+__global__ __launch_bounds__(1024) void sort_scan_kernel(int E, int nblk, int32_t* __restrict__ ws,
+                                                         int32_t* __restrict__ expert_offsets) {
+  __shared__ int totals[SORT_MAX_E];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int e = wave; e < E; e += 16) {
+    int32_t* row = ws + (size_t)e * nblk;
+    int carry = 0;
+    for (int b0 = 0; b0 < nblk; b0 += 64) {
+      int b = b0 + lane;
+      int v = b < nblk ? row[b] : 0;
+      int inc = wave_incl_scan_i32(v, lane);
+      if (b < nblk) row[b] = carry + inc - v;
+      carry += __shfl(inc, 63, MI_WAVE);
+    }
+    if (lane == 0) totals[e] = carry;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    int carry = 0;
+    int32_t* ebase = ws + (size_t)E * nblk;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      int e = e0 + lane;
+      int v = e < E ? totals[e] : 0;
+      int inc = wave_incl_scan_i32(v, lane);
+      if (e < E) {
+        expert_offsets[e] = carry + inc;
+        ebase[e] = carry + inc - v;
+      }
+      carry += __shfl(inc, 63, MI_WAVE);
+    }
+  }
+}
+
+// Stable scatter of one chunk [chunk_begin, chunk_end).  wbase[w * E + e] must hold, on entry, the
+// output position of the first slot of expert e seen by wave w.
+__device__ __forceinline__ void sort_scatter_chunk(const int32_t* __restrict__ ids, int chunk_begin, int chunk_end,
+                                                   int per_wave, int E, int nbits, int* wbase,
+                                                   int32_t* __restrict__ sorted_expert,
+                                                   int32_t* __restrict__ sorted_scattered) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int* mybase = wbase + wave * E;
+  const int begin = chunk_begin + wave * per_wave;
+  int end = begin + per_wave;
+  if (end > chunk_end) end = chunk_end;
+  for (int s0 = begin; s0 < end; s0 += 64) {
+    const int slot = s0 + lane;
+    const bool valid = slot < end;
+    int e = valid ? ids[slot] : 0;
+    const bool ok = valid && (unsigned)e < (unsigned)E;
+    if (!ok) e = 0;
+    uint64_t peers = __ballot(ok);
+    for (int b = 0; b < nbits; ++b) {
+      uint64_t bal = __ballot((e >> b) & 1);
+      peers &= ((e >> b) & 1) ? bal : ~bal;
+    }
+    if (ok) {
+      const uint64_t below = peers & ((1ull << lane) - 1ull);
+      const int rank = __popcll(below);
+      const int pos = mybase[e] + rank;
+      sorted_expert[pos] = e;
+      sorted_scattered[pos] = slot;
+      // every lane of the group has read mybase[e] (one LDS instruction, wave-wide) before the
+      // group's first lane bumps it for the next step
+      if (below == 0ull) mybase[e] += __popcll(peers);
+    }
+  }
+}
+
+// Per-wave histograms of a chunk into wcnt[w * E + e] (LDS, pre-zeroed).
+__device__ __forceinline__ void sort_wave_hist(const int32_t* __restrict__ ids, int chunk_begin, int chunk_end,
+                                               int per_wave, int E, int* wcnt) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int begin = chunk_begin + wave * per_wave;
+  int end = begin + per_wave;
+  if (end > chunk_end) end = chunk_end;
+  for (int s = begin + lane; s < end; s += 64) {
+    int e = ids[s];
+    if ((unsigned)e < (unsigned)E) atomicAdd(&wcnt[wave * E + e], 1);
+  }
+}
+
+__global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(const int32_t* __restrict__ ids, int L, int E,
+                                                                    int nbits, int nblk,
+                                                                    const int32_t* __restrict__ ws,
+                                                                    int32_t* __restrict__ sorted_expert,
+                                                                    int32_t* __restrict__ sorted_scattered) {
+  extern __shared__ int wcnt[];  // SORT_WAVES * E
+  for (int i = threadIdx.x; i < SORT_WAVES * E; i += SORT_THREADS) wcnt[i] = 0;
+  __syncthreads();
+  const int chunk_begin = blockIdx.x * SORT_CHUNK;
+  int chunk_end = chunk_begin + SORT_CHUNK;
+  if (chunk_end > L) chunk_end = L;
+  const int per_wave = SORT_CHUNK / SORT_WAVES;
+  sort_wave_hist(ids, chunk_begin, chunk_end, per_wave, E, wcnt);
+  __syncthreads();
+  const int32_t* ebase = ws + (size_t)E * nblk;
+  for (int e = threadIdx.x; e < E; e += SORT_THREADS) {
+    int run = ws[(size_t)e * nblk + blockIdx.x] + ebase[e];
+#pragma unroll
+    for (int w = 0; w < SORT_WAVES; ++w) {
+      int c = wcnt[w * E + e];
+      wcnt[w * E + e] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+  sort_scatter_chunk(ids, chunk_begin, chunk_end, per_wave, E, nbits, wcnt, sorted_expert, sorted_scattered);
+}
+
+// Whole problem in one block: histogram, expert scan and scatter without touching a workspace.
+__global__ __launch_bounds__(SORT_THREADS) void sort_single_block_kernel(const int32_t* __restrict__ ids, int L,
+                                                                         int E, int nbits,
+                                                                         int32_t* __restrict__ sorted_expert,
+                                                                         int32_t* __restrict__ sorted_scattered,
+                                                                         int32_t* __restrict__ expert_offsets) {
+  extern __shared__ int smem[];  // SORT_WAVES * E counters, then E totals
+  int* wcnt = smem;
+  int* totals = smem + SORT_WAVES * E;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < SORT_WAVES * E; i += SORT_THREADS) wcnt[i] = 0;
+  __syncthreads();
+  const int per_wave = mi_ceil_div_dev(mi_ceil_div_dev(L, SORT_WAVES), 64) * 64;
+  sort_wave_hist(ids, 0, L, per_wave, E, wcnt);
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += SORT_THREADS) {
+    int t = 0;
+#pragma unroll
+    for (int w = 0; w < SORT_WAVES; ++w) t += wcnt[w * E + e];
+    totals[e] = t;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    int carry = 0;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      int e = e0 + lane;
+      int v = e < E ? totals[e] : 0;
+      int inc = wave_incl_scan_i32(v, lane);
+      if (e < E) {
+        expert_offsets[e] = carry + inc;
+        totals[e] = carry + inc - v;  // exclusive base
+      }
+      carry += __shfl(inc, 63, MI_WAVE);
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += SORT_THREADS) {
+    int run = totals[e];
+#pragma unroll
+    for (int w = 0; w < SORT_WAVES; ++w) {
+      int c = wcnt[w * E + e];
+      wcnt[w * E + e] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+  sort_scatter_chunk(ids, 0, L, per_wave, E, nbits, wcnt, sorted_expert, sorted_scattered);
+}
+
+#define SORT_SINGLE_BLOCK_MAX 8192
+
+extern "C" size_t mi_moe_sort_bin_workspace_bytes(int L, int E) {
+  if (L <= SORT_SINGLE_BLOCK_MAX || E < 1) return 0;
+  size_t nblk = (size_t)mi_ceil_div(L, SORT_CHUNK);
+  return ((size_t)E * nblk + (size_t)E) * sizeof(int32_t);
+}
+
+extern "C" int mi_moe_sort_bin(const int32_t* topk_idx, int T, int k, int E, int32_t* sorted_expert,
+                               int32_t* sorted_scattered, int32_t* expert_offsets, void* ws, size_t ws_bytes,
+                               mi_moe_stream_t stream) {
+  if (T < 0 || k < 1 || E < 1 || E > SORT_MAX_E) return MI_MOE_ESHAPE;
+  if ((int64_t)T * k > (int64_t)0x7fffffff - SORT_CHUNK) return MI_MOE_ESHAPE;
+  if (!expert_offsets) return MI_MOE_ENULL;
+  const int L = T * k;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (L > 0 && (!topk_idx || !sorted_expert || !sorted_scattered)) return MI_MOE_ENULL;
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  if (L <= SORT_SINGLE_BLOCK_MAX) {
+    size_t lds = (size_t)(SORT_WAVES + 1) * E * sizeof(int);
+    hipLaunchKernelGGL(sort_single_block_kernel, dim3(1), dim3(SORT_THREADS), lds, s, topk_idx, L, E, nbits,
+                       sorted_expert, sorted_scattered, expert_offsets);
+    return mi_launch_status();
+  }
+  const int nblk = mi_ceil_div(L, SORT_CHUNK);
+  if (ws_bytes < mi_moe_sort_bin_workspace_bytes(L, E) || !ws) return MI_MOE_EWORKSPACE;
+  if (!mi_aligned(ws, 16)) return MI_MOE_EALIGN;
+  int32_t* w = static_cast<int32_t*>(ws);
+  hipLaunchKernelGGL(sort_hist_kernel, dim3(nblk), dim3(SORT_THREADS), 0, s, topk_idx, L, E, nblk, w);
+  hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(1024), 0, s, E, nblk, w, expert_offsets);
+  size_t lds = (size_t)SORT_WAVES * E * sizeof(int);
+  hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblk), dim3(SORT_THREADS), lds, s, topk_idx, L, E, nbits, nblk, w,
+                     sorted_expert, sorted_scattered);
+  return mi_launch_status();
+}

@@ -1,0 +1,382 @@
+"""MoE layer with the scattered-expert forward on MI355X.
+
+Same constructor, attributes, state-dict names/shapes and forward contract as the reference's
+``MoE`` / ``ParameterizedExperts`` (lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:48-384):
+
+    gate.weight   (E, H)
+    c_fc.weight   (E, 2I, H) for a GLU activation ([up ; gate] rows), else (E, I, H)
+    c_proj.weight (E, H, I)
+    (+ c_fc_shared / c_proj_shared when shared_intermediate_size is given)
+
+With ``enable_kernels([Kernel.scattermoe])`` the expert computation runs on the HIP kernels of
+this package (router -> sort/bin -> grouped up-projection with fused SwiGLU -> grouped
+down-projection -> gate-weighted combine).  Without it the eager torch branch runs, which is the
+reference's own eager branch (moe.py:292-307) and works on any device.
+
+The kernel branch is forward-only (inference): it refuses tensors that require grad while grad
+mode is on, and it raises if the kernel library is missing -- it never falls back silently.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+from .activations import GLUActivation, get_activation_function, is_glu
+from .enums import Kernel
+from .kernels import is_kernel_allowed
+from .linear import ParameterizedLinear
+from .loss import add_aux_loss
+from .parameter import mark_parameter_as_mup_learning_rate, mark_parameter_as_no_weight_decay
+
+
+def _get_std_for_linear(initializer_range: float, init_method: str, m_width: float | None) -> float:
+    """lm_engine/hf_models/modeling_utils/mlp_blocks/mlp.py:58-65."""
+    std = initializer_range
+    if init_method == "mup":
+        std /= math.sqrt(m_width)
+    elif init_method != "normal":
+        raise ValueError(f"unexpected init_method ({init_method})")
+    return std
+
+
+def bincount(x: torch.Tensor, minlength: int) -> torch.Tensor:
+    """moe.py:27-30."""
+    return x.bincount(minlength=minlength).to(torch.uint32)
+
+
+def compute_bincount(x: torch.Tensor, size: int, use_continuous_count: bool) -> torch.Tensor:
+    """moe.py:38-44: the HIP histogram when asked for, else torch.bincount."""
+    if use_continuous_count:
+        return ops.continuous_count(x, size=size)
+    return bincount(x, minlength=size)
+
+
+class ParameterizedExperts(nn.Module):
+    """E stacked linear layers, weight (E, out, in) (moe.py:48-121)."""
+
+    def __init__(self, num_experts: int, in_features: int, out_features: int, add_bias: bool = True,
+                 device=None, dtype=None, std: float | None = None) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(num_experts, out_features, in_features, device=device, dtype=dtype))
+        self.bias = None
+        if add_bias:
+            self.bias = nn.Parameter(torch.empty(num_experts, out_features, device=device, dtype=dtype))
+        self.std = std
+        self.num_experts = num_experts
+        self.in_features = in_features
+        self.out_features = out_features
+        # optional fp8 storage (see MoE.quantize_expert_weights_fp8)
+        self.weight_scale_dtype = None
+        self.register_buffer("weight_q", None, persistent=True)
+        self.register_buffer("weight_scale", None, persistent=True)
+        self.reset_parameters()
+        mark_parameter_as_no_weight_decay(self.bias)
+
+    def dense_weight(self) -> torch.Tensor:
+        """The (E, out, in) weight the eager branch multiplies with (dequantised if stored as fp8)."""
+        if self.weight_q is not None:
+            return (self.weight_q.float() * self.weight_scale.unsqueeze(-1)).to(self.weight_scale_dtype)
+        return self.weight
+
+    def forward(self, input: torch.Tensor, num_experts_per_token: int | None = None,
+                num_tokens_per_expert: torch.Tensor | None = None,
+                sorted_expert_idxs: torch.Tensor | None = None, sorted_scattered_idxs: torch.Tensor | None = None,
+                expert_offsets: torch.Tensor | None = None, gates: torch.Tensor | None = None,
+                grouped_in: bool = False, grouped_out: bool = False) -> torch.Tensor:
+        if is_kernel_allowed(Kernel.scattermoe):
+            assert self.bias is None
+            if self.weight_q is not None:
+                raise RuntimeError("fp8 expert weights are only supported through MoE.forward")
+            return ops.scattered_experts(
+                inputs=input,
+                expert_weights=self.weight.permute(0, 2, 1),
+                k=num_experts_per_token,
+                sorted_expert_idxs=sorted_expert_idxs,
+                sorted_scattered_idxs=sorted_scattered_idxs,
+                expert_offsets=expert_offsets,
+                gates=gates,
+                grouped_in=grouped_in,
+                grouped_out=grouped_out,
+            )
+        weight = self.dense_weight()
+        pieces = input.split(num_tokens_per_expert.tolist(), dim=0)
+        outs = [
+            F.linear(pieces[i], weight[i].to(input.dtype), None if self.bias is None else self.bias[i])
+            for i in range(self.num_experts)
+        ]
+        return torch.cat(outs, dim=0)
+
+    def extra_repr(self) -> str:
+        return "num_experts={}, in_features={}, out_features={}".format(
+            self.num_experts, self.in_features, self.out_features
+        )
+
+    @torch.no_grad()
+    def reset_parameters(self) -> None:
+        nn.init.normal_(self.weight, mean=0, std=self.std)
+        if getattr(self, "bias", None) is not None:
+            self.bias.zero_()
+
+    @torch.no_grad()
+    def quantize_fp8(self) -> None:
+        """Replace the weight by e4m3fn values plus one fp32 scale per output channel
+        (scale = max|row| / 448)."""
+        w = self.weight.detach().float()
+        scale = w.abs().amax(dim=-1).clamp_min(1e-12) / 448.0
+        self.weight_scale_dtype = self.weight.dtype
+        self.weight_q = (w / scale.unsqueeze(-1)).to(torch.float8_e4m3fn)
+        self.weight_scale = scale
+        self.weight = None
+
+
+class MoE(nn.Module):
+    linear_class = ParameterizedExperts
+
+    def __init__(self, hidden_size: int, intermediate_size: int, shared_intermediate_size: int | None,
+                 num_experts: int, num_experts_per_tok: int, activation_function: str, add_bias: bool,
+                 dropout: float, init_method: str, initializer_range: float, m_width: float | None,
+                 num_layers: int, use_padding_free_transformer: bool) -> None:
+        super().__init__()
+
+        self.num_experts = num_experts
+        self.top_k = num_experts_per_tok
+        self.use_padding_free_transformer = use_padding_free_transformer
+
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.shared_intermediate_size = shared_intermediate_size
+
+        std = _get_std_for_linear(initializer_range, init_method, m_width)
+        glu = is_glu(activation_function)
+
+        self.gate = ParameterizedLinear(in_features=hidden_size, out_features=num_experts, bias=False, std=std)
+        self.c_fc = self.linear_class(
+            num_experts=num_experts,
+            in_features=hidden_size,
+            out_features=2 * intermediate_size if glu else intermediate_size,
+            add_bias=add_bias,
+            std=std,
+        )
+        if shared_intermediate_size is not None:
+            self.c_fc_shared = ParameterizedLinear(
+                in_features=hidden_size,
+                out_features=2 * shared_intermediate_size if glu else shared_intermediate_size,
+                bias=add_bias,
+                std=std,
+            )
+
+        self.act = get_activation_function(activation_function)
+        self._fused_swiglu = isinstance(self.act, GLUActivation) and isinstance(self.act.base_activation, nn.SiLU)
+
+        std /= math.sqrt(2 * num_layers)
+
+        self.c_proj = self.linear_class(
+            num_experts=num_experts, in_features=intermediate_size, out_features=hidden_size, add_bias=add_bias,
+            std=std,
+        )
+        if shared_intermediate_size is not None:
+            self.c_proj_shared = ParameterizedLinear(
+                in_features=shared_intermediate_size, out_features=hidden_size, bias=add_bias, std=std
+            )
+
+        self.dropout = nn.Identity() if dropout == 0 else nn.Dropout(dropout)
+
+        # benchmark-input construct: an optional per-expert offset added to the router logits
+        # before top-k (skews the expert load); None reproduces the reference exactly
+        self.register_buffer("router_logit_bias", None, persistent=False)
+
+        mark_parameter_as_mup_learning_rate(self.gate.weight)
+        mark_parameter_as_mup_learning_rate(self.c_fc.weight)
+        mark_parameter_as_mup_learning_rate(self.c_proj.weight)
+        if shared_intermediate_size is not None:
+            mark_parameter_as_mup_learning_rate(self.c_fc_shared.weight)
+            mark_parameter_as_mup_learning_rate(self.c_proj_shared.weight)
+
+    # ---------------------------------------------------------------------------------------------
+
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        if not self.use_padding_free_transformer:
+            batch_size, sequence_length, _ = hidden_states.shape
+
+        hidden_states = hidden_states.view(-1, self.hidden_size)
+
+        router_logits, router_weights, selected_experts = self._compute_routing_weights(hidden_states)
+        moe_output = self._compute_experts(hidden_states, router_weights, selected_experts)
+
+        if self.shared_intermediate_size is None:
+            hidden_states = moe_output
+        else:
+            hidden_states = moe_output + self._compute_shared_experts(hidden_states)
+        del moe_output
+
+        if not self.use_padding_free_transformer:
+            hidden_states = hidden_states.reshape(batch_size, sequence_length, self.hidden_size)
+
+        hidden_states = self.dropout(hidden_states)
+
+        aux_loss = (
+            self._compute_switch_loss(
+                logits=router_logits, probs=torch.softmax(router_logits, dim=-1), topk_idxs=selected_experts
+            )
+            if self.training
+            else 0
+        )
+        add_aux_loss(aux_loss)
+
+        return hidden_states
+
+    def _use_fused_router(self, hidden_states: torch.Tensor) -> bool:
+        return (
+            is_kernel_allowed(Kernel.scattermoe)
+            and not self.training
+            and hidden_states.is_cuda
+            and ops.router_fused_supported(hidden_states, self.num_experts, self.top_k)
+        )
+
+    def _compute_routing_weights(self, hidden_states: torch.Tensor):
+        """moe.py:246-257.  On the kernel path in eval mode the gate GEMM, top-k and softmax are one
+        kernel and the (T, E) logits are never written (only the training aux loss reads them)."""
+        if self._use_fused_router(hidden_states):
+            _, router_weights, selected_experts = ops.router_fused(
+                hidden_states, self.gate.weight, self.top_k, bias=self.router_logit_bias
+            )
+            return None, router_weights, selected_experts
+
+        router_logits = self.gate(hidden_states)
+        if self.router_logit_bias is not None:
+            router_logits = (router_logits.float() + self.router_logit_bias.float()).to(router_logits.dtype)
+
+        if is_kernel_allowed(Kernel.scattermoe) and hidden_states.is_cuda and not torch.is_grad_enabled():
+            router_weights, selected_experts = ops.router_topk_softmax(router_logits, self.top_k)
+        else:
+            router_weights, selected_experts = self._get_topk(router_logits)
+            router_weights = F.softmax(router_weights.float(), dim=-1)
+            router_weights = router_weights.type_as(hidden_states)
+
+        return router_logits, router_weights, selected_experts
+
+    def _compute_experts(self, hidden_states: torch.Tensor, router_weights: torch.Tensor,
+                         selected_experts: torch.Tensor) -> torch.Tensor:
+        if is_kernel_allowed(Kernel.scattermoe):
+            sorted_expert_idxs, sorted_scattered_idxs, expert_offsets = ops.sort_bin(selected_experts, self.num_experts)
+
+            if self.c_fc.weight_q is not None:
+                if not self._fused_swiglu:
+                    raise RuntimeError("fp8 expert weights need the swiglu activation")
+                hidden_states = ops.up_swiglu_fp8(hidden_states, self.c_fc.weight_q, self.c_fc.weight_scale,
+                                                  self.top_k, sorted_scattered_idxs, expert_offsets)
+                hidden_states = ops.down_fp8(hidden_states, self.c_proj.weight_q, self.c_proj.weight_scale,
+                                             sorted_scattered_idxs, expert_offsets)
+                hidden_states = ops.combine(hidden_states, router_weights)
+            else:
+                if self._fused_swiglu:
+                    assert self.c_fc.bias is None
+                    hidden_states = ops.up_swiglu(hidden_states, self.c_fc.weight, self.top_k,
+                                                  sorted_scattered_idxs, expert_offsets)
+                else:
+                    hidden_states = self.c_fc(
+                        input=hidden_states,
+                        num_experts_per_token=self.top_k,
+                        sorted_expert_idxs=sorted_expert_idxs,
+                        sorted_scattered_idxs=sorted_scattered_idxs,
+                        expert_offsets=expert_offsets,
+                        grouped_out=True,
+                    )
+                    hidden_states = self.act(hidden_states)
+                hidden_states = self.c_proj(
+                    input=hidden_states,
+                    num_experts_per_token=1,
+                    sorted_expert_idxs=sorted_expert_idxs,
+                    sorted_scattered_idxs=sorted_scattered_idxs,
+                    expert_offsets=expert_offsets,
+                    grouped_in=True,
+                    gates=router_weights,
+                )
+            hidden_states = self.dropout(hidden_states)
+        else:
+            total_q = hidden_states.shape[0]
+
+            batch_index, batch_gates, num_tokens_per_expert = self._compute_expert_assignment(
+                router_weights, selected_experts
+            )
+
+            hidden_states = hidden_states[batch_index]
+            hidden_states = self.c_fc(input=hidden_states, num_tokens_per_expert=num_tokens_per_expert)
+            hidden_states = self.act(hidden_states)
+            hidden_states = self.c_proj(input=hidden_states, num_tokens_per_expert=num_tokens_per_expert)
+
+            hidden_states = hidden_states * batch_gates.unsqueeze(-1)
+            zeros = torch.zeros((total_q, self.hidden_size), dtype=hidden_states.dtype, device=hidden_states.device)
+            hidden_states = zeros.index_add(0, batch_index, hidden_states)
+
+        return hidden_states
+
+    def _compute_shared_experts(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        hidden_states = self.c_fc_shared(hidden_states)
+        hidden_states = self.act(hidden_states)
+        hidden_states = self.c_proj_shared(hidden_states)
+        return hidden_states
+
+    def _compute_expert_assignment(self, router_weights: torch.Tensor, selected_experts: torch.Tensor):
+        """moe.py:317-336 (stable sort: within-expert order is then defined)."""
+        selected_experts = selected_experts.flatten().long()
+        num_tokens_per_expert = compute_bincount(
+            x=selected_experts, size=self.num_experts,
+            use_continuous_count=selected_experts.is_cuda and is_kernel_allowed(Kernel.continuous_count_cute),
+        )
+        _, index_sorted_experts = selected_experts.sort(stable=True)
+        batch_index = index_sorted_experts // self.top_k
+        batch_gates = router_weights.flatten()[index_sorted_experts]
+        return batch_index, batch_gates, num_tokens_per_expert
+
+    def _get_topk(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        """moe.py:338-344."""
+        if self.top_k == 1:
+            x, indices = x.max(dim=-1, keepdim=True)
+        else:
+            x, indices = x.topk(self.top_k, dim=-1)
+        return x, indices
+
+    def _compute_switch_loss(self, logits: torch.Tensor, probs: torch.Tensor, topk_idxs: torch.Tensor) -> torch.Tensor:
+        """moe.py:346-369 for a single data-parallel rank."""
+        logits = logits.view(-1, logits.size(-1))
+        probs = probs.view(-1, probs.size(-1))
+
+        num_experts = logits.size(1)
+        acc_probs = probs.sum(0)
+        freq = compute_bincount(
+            x=topk_idxs.flatten().long(), size=num_experts,
+            use_continuous_count=topk_idxs.is_cuda and is_kernel_allowed(Kernel.continuous_count_cute),
+        ).float()
+
+        switch_loss = num_experts * (F.normalize(acc_probs, p=1, dim=0) * F.normalize(freq, p=1, dim=0)).sum()
+        z_loss = (torch.logsumexp(logits, dim=-1) ** 2).mean()
+        loss = switch_loss + 0.1 * z_loss
+        return loss.type_as(logits)
+
+    def get_num_active_parameters(self) -> int:
+        """moe.py:371-384."""
+        num_elements = 0
+        for parameter in self.parameters():
+            num_elements += parameter.numel()
+        for parameter in self.c_fc.parameters():
+            num_elements -= parameter.numel()
+            num_elements += (parameter.numel() * self.top_k) // self.num_experts
+        for parameter in self.c_proj.parameters():
+            num_elements -= parameter.numel()
+            num_elements += (parameter.numel() * self.top_k) // parameter.size(0)
+        return num_elements
+
+    @torch.no_grad()
+    def quantize_expert_weights_fp8(self) -> None:
+        """Store c_fc / c_proj as e4m3fn + per-output-channel fp32 scales (decode-shape serving).
+        Not part of the reference; the eager branch then multiplies with the dequantised weights."""
+        if self.c_fc.bias is not None or self.c_proj.bias is not None:
+            raise RuntimeError("fp8 expert weights do not support biases")
+        self.c_fc.quantize_fp8()
+        self.c_proj.quantize_fp8()

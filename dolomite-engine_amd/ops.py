@@ -1,0 +1,312 @@
+"""Tensor-level wrappers over the C ABI (include/mi_moe.h).
+
+``scattered_experts`` and ``continuous_count`` keep the call signatures the reference uses for the
+external ops it imports at lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:22-24 (call sites
+moe.py:40 and moe.py:91-101), so either can be bound in their place.  The remaining functions are
+the fused stages the MoE module of this package calls.
+
+PyTorch is used for device memory and the current stream only; every function enqueues HIP
+kernels on ``torch.cuda.current_stream()`` and returns without synchronising.  All of this is
+forward-only: tensors that require grad are refused while grad mode is on.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import BF16, F16, F32, check
+
+_DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+
+
+_TIMER = None
+
+
+def set_stage_timer(timer) -> None:
+    """Install an object with ``begin(name)`` / ``end(name)`` that is called around every kernel
+    stage (used by the benchmark to put HIP events on the launch stream); ``None`` removes it."""
+    global _TIMER
+    _TIMER = timer
+
+
+class _stage:
+    def __init__(self, name: str):
+        self.name = name
+
+    def __enter__(self):
+        if _TIMER is not None:
+            _TIMER.begin(self.name)
+
+    def __exit__(self, *exc):
+        if _TIMER is not None:
+            _TIMER.end(self.name)
+        return False
+
+
+def is_available() -> bool:
+    """True when a GPU is visible and the kernel library has been built."""
+    return torch.cuda.is_available() and _lib.is_built()
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dtype} (float32, float16 and bfloat16 are supported)") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(*tensors: torch.Tensor | None) -> None:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("the scattermoe kernels need tensors on the GPU (no CPU fallback)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ValueError("all tensors must be on the same device")
+    if dev is not None and dev.index is not None and dev.index != torch.cuda.current_device():
+        raise ValueError("tensors must be on the current device")
+
+
+def _no_grad(*tensors: torch.Tensor | None) -> None:
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise RuntimeError(
+            "the MI355X scattermoe kernels are forward-only: run under torch.no_grad() / inference_mode()"
+        )
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _i32(t: torch.Tensor) -> torch.Tensor:
+    return t if t.dtype == torch.int32 else t.to(torch.int32)
+
+
+def _native_weight(expert_weights: torch.Tensor) -> torch.Tensor:
+    """(E, in, out) view as passed by the reference -> contiguous (E, out, in) storage, without a copy
+    when the argument is the permuted view of the module's parameter."""
+    w = expert_weights.permute(0, 2, 1)
+    return w if w.is_contiguous() else w.contiguous()
+
+
+# ------------------------------------------------------------------------------------------------
+# routing
+# ------------------------------------------------------------------------------------------------
+
+
+def router_topk_softmax(logits: torch.Tensor, k: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Top-k (value descending, expert index ascending) + fp32 softmax over the k values.
+
+    logits (T, E) -> gates (T, k) in logits.dtype, experts (T, k) int32."""
+    _dev(logits)
+    _no_grad(logits)
+    logits = logits.contiguous()
+    T, E = logits.shape
+    gates = torch.empty((T, k), dtype=logits.dtype, device=logits.device)
+    idx = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+    with _stage("router_topk_softmax"):
+        check(_lib.load().mi_moe_router_topk_softmax(_ptr(logits), T, E, k, _code(logits.dtype), _ptr(gates), _ptr(idx),
+                                                    _stream()))
+    return gates, idx
+
+
+def router_fused_supported(x: torch.Tensor, num_experts: int, k: int) -> bool:
+    return (x.dtype in (torch.bfloat16, torch.float16) and num_experts <= 64 and k <= 8 and x.shape[-1] % 16 == 0)
+
+
+def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch.Tensor | None = None,
+                 return_logits: bool = False):
+    """logits = x @ gate_weight^T (+bias) in x.dtype, top-k, softmax: one pass over x.
+
+    Returns (logits or None, gates (T,k), experts (T,k) int32)."""
+    _dev(x, gate_weight, bias)
+    _no_grad(x, gate_weight)
+    x = x.contiguous()
+    gate_weight = gate_weight.contiguous()
+    T, H = x.shape
+    E = gate_weight.shape[0]
+    if gate_weight.dtype != x.dtype or gate_weight.shape[1] != H:
+        raise ValueError("gate weight must be (E, H) in the dtype of x")
+    if bias is not None:
+        bias = bias.to(torch.float32).contiguous()
+    logits = torch.empty((T, E), dtype=x.dtype, device=x.device) if return_logits else None
+    gates = torch.empty((T, k), dtype=x.dtype, device=x.device)
+    idx = torch.empty((T, k), dtype=torch.int32, device=x.device)
+    with _stage("router_fused"):
+        check(_lib.load().mi_moe_router_fused(_ptr(x), _ptr(gate_weight), _ptr(bias), T, H, E, k, _code(x.dtype),
+                                             _ptr(logits), _ptr(gates), _ptr(idx), _stream()))
+    return logits, gates, idx
+
+
+def continuous_count(x: torch.Tensor, size: int) -> torch.Tensor:
+    """Histogram of the integer tensor ``x`` with ``size`` bins, uint32 (moe.py:38-44)."""
+    _dev(x)
+    ids = _i32(x.flatten()).contiguous()
+    out = torch.empty(size, dtype=torch.uint32, device=x.device)
+    with _stage("count"):
+        check(_lib.load().mi_moe_count(_ptr(ids), ids.numel(), size, _ptr(out), _stream()))
+    return out
+
+
+def sort_bin(selected_experts: torch.Tensor, num_experts: int):
+    """Stable expert sort + inclusive offsets (moe.py:263-271).
+
+    selected_experts (T, k) integer -> (sorted_expert_idxs (L,), sorted_scattered_idxs (L,),
+    expert_offsets (E,)), all int32."""
+    _dev(selected_experts)
+    T, k = selected_experts.shape
+    ids = _i32(selected_experts).contiguous()
+    L = T * k
+    dev = ids.device
+    se = torch.empty(L, dtype=torch.int32, device=dev)
+    ss = torch.empty(L, dtype=torch.int32, device=dev)
+    off = torch.empty(num_experts, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    ws_bytes = lib.mi_moe_sort_bin_workspace_bytes(L, num_experts)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    with _stage("sort_bin"):
+        check(lib.mi_moe_sort_bin(_ptr(ids), T, k, num_experts, _ptr(se), _ptr(ss), _ptr(off), _ptr(ws), ws_bytes,
+                                  _stream()))
+    return se, ss, off
+
+
+# ------------------------------------------------------------------------------------------------
+# experts
+# ------------------------------------------------------------------------------------------------
+
+
+def scattered_gemm(inputs: torch.Tensor, weight: torch.Tensor, k: int, sorted_scattered_idxs: torch.Tensor,
+                   expert_offsets: torch.Tensor, grouped_in: bool, grouped_out: bool, cfg: int = -1) -> torch.Tensor:
+    """Grouped GEMM with the weight in native (E, out, in) layout; returns (L, out)."""
+    _dev(inputs, weight, sorted_scattered_idxs, expert_offsets)
+    _no_grad(inputs, weight)
+    inputs = inputs.contiguous()
+    weight = weight.contiguous()
+    ss = _i32(sorted_scattered_idxs).contiguous()
+    off = _i32(expert_offsets).contiguous()
+    E, N, K = weight.shape
+    if inputs.shape[1] != K or weight.dtype != inputs.dtype:
+        raise ValueError("inputs must be (rows, in_features) in the dtype of the weights")
+    L = ss.numel()
+    if grouped_in and inputs.shape[0] != L:
+        raise ValueError("grouped inputs must have one row per sorted slot")
+    if not grouped_in and inputs.shape[0] * k != L:
+        raise ValueError("scattered inputs must have L / k rows")
+    out = torch.empty((L, N), dtype=inputs.dtype, device=inputs.device)
+    with _stage("scattered_gemm"):
+        check(_lib.load().mi_moe_scattered_gemm_cfg(_ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N,
+                                                   E, k, int(grouped_in), int(grouped_out), _code(inputs.dtype), cfg,
+                                                   _stream()))
+    return out
+
+
+def combine(o: torch.Tensor, gates: torch.Tensor) -> torch.Tensor:
+    """y[t] = sum_j gates[t, j] * o[t*k + j]  with o (T*k, H), gates (T, k)."""
+    _dev(o, gates)
+    _no_grad(o, gates)
+    o = o.contiguous()
+    gates = gates.contiguous()
+    T, k = gates.shape
+    H = o.shape[1]
+    if o.shape[0] != T * k or gates.dtype != o.dtype:
+        raise ValueError("o must be (T*k, H) and gates (T, k) of the same dtype")
+    y = torch.empty((T, H), dtype=o.dtype, device=o.device)
+    with _stage("combine"):
+        check(_lib.load().mi_moe_combine(_ptr(o), _ptr(gates), _ptr(y), T, k, H, _code(o.dtype), _stream()))
+    return y
+
+
+def scattered_experts(inputs: torch.Tensor, expert_weights: torch.Tensor, k: int,
+                      sorted_expert_idxs: torch.Tensor, sorted_scattered_idxs: torch.Tensor,
+                      expert_offsets: torch.Tensor, gates: torch.Tensor | None = None, grouped_in: bool = False,
+                      grouped_out: bool = False) -> torch.Tensor:
+    """Drop-in for the external ``scattered_experts`` (moe.py:91-101).
+
+    ``expert_weights`` is the (E, in, out) view the reference passes (``weight.permute(0, 2, 1)``);
+    ``sorted_expert_idxs`` is accepted for signature compatibility (the kernels derive the expert of
+    a row from ``expert_offsets``).  With ``gates`` (T, k_g) the (L, out) result is contracted to
+    (T, out)."""
+    del sorted_expert_idxs
+    w = _native_weight(expert_weights)
+    if gates is not None and grouped_out:
+        raise ValueError("gates need the output in flat-slot order (grouped_out=False)")
+    out = scattered_gemm(inputs, w, k, sorted_scattered_idxs, expert_offsets, grouped_in, grouped_out)
+    if gates is not None:
+        out = combine(out, gates.to(out.dtype))
+    return out
+
+
+def up_swiglu(x: torch.Tensor, w_fc: torch.Tensor, k: int, sorted_scattered_idxs: torch.Tensor,
+              expert_offsets: torch.Tensor, cfg: int = -1) -> torch.Tensor:
+    """Up-projection with SwiGLU fused: x (T, H), w_fc (E, 2I, H) -> (L, I) in grouped order."""
+    _dev(x, w_fc, sorted_scattered_idxs, expert_offsets)
+    _no_grad(x, w_fc)
+    x = x.contiguous()
+    w_fc = w_fc.contiguous()
+    ss = _i32(sorted_scattered_idxs).contiguous()
+    off = _i32(expert_offsets).contiguous()
+    E, I2, H = w_fc.shape
+    if x.shape[1] != H or w_fc.dtype != x.dtype or I2 % 2:
+        raise ValueError("x must be (T, H), w_fc (E, 2I, H), same dtype")
+    L = ss.numel()
+    if x.shape[0] * k != L:
+        raise ValueError("x must have L / k rows")
+    act = torch.empty((L, I2 // 2), dtype=x.dtype, device=x.device)
+    with _stage("up_swiglu"):
+        check(_lib.load().mi_moe_up_swiglu_cfg(_ptr(x), _ptr(w_fc), _ptr(act), _ptr(ss), _ptr(off), L, H, I2 // 2, E, k,
+                                              _code(x.dtype), cfg, _stream()))
+    return act
+
+
+def up_swiglu_fp8(x: torch.Tensor, w_fc_q: torch.Tensor, w_fc_scale: torch.Tensor, k: int,
+                  sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor) -> torch.Tensor:
+    """As up_swiglu with e4m3fn weights (E, 2I, H) and fp32 per-output-channel scales (E, 2I)."""
+    _dev(x, w_fc_q, w_fc_scale, sorted_scattered_idxs, expert_offsets)
+    _no_grad(x)
+    if w_fc_q.dtype != torch.float8_e4m3fn:
+        raise TypeError("weights must be torch.float8_e4m3fn")
+    x = x.contiguous()
+    w_fc_q = w_fc_q.contiguous()
+    scale = w_fc_scale.to(torch.float32).contiguous()
+    ss = _i32(sorted_scattered_idxs).contiguous()
+    off = _i32(expert_offsets).contiguous()
+    E, I2, H = w_fc_q.shape
+    L = ss.numel()
+    if x.shape[1] != H or x.shape[0] * k != L or scale.shape != (E, I2):
+        raise ValueError("shape mismatch")
+    act = torch.empty((L, I2 // 2), dtype=x.dtype, device=x.device)
+    with _stage("up_swiglu_fp8"):
+        check(_lib.load().mi_moe_up_swiglu_fp8(_ptr(x), _ptr(w_fc_q), _ptr(scale), _ptr(act), _ptr(ss), _ptr(off), L, H,
+                                              I2 // 2, E, k, _code(x.dtype), _stream()))
+    return act
+
+
+def down_fp8(act: torch.Tensor, w_proj_q: torch.Tensor, w_proj_scale: torch.Tensor,
+             sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor) -> torch.Tensor:
+    """Down-projection with e4m3fn weights (E, H, I): act (L, I) grouped -> (L, H) in flat-slot order."""
+    _dev(act, w_proj_q, w_proj_scale, sorted_scattered_idxs, expert_offsets)
+    _no_grad(act)
+    if w_proj_q.dtype != torch.float8_e4m3fn:
+        raise TypeError("weights must be torch.float8_e4m3fn")
+    act = act.contiguous()
+    w_proj_q = w_proj_q.contiguous()
+    scale = w_proj_scale.to(torch.float32).contiguous()
+    ss = _i32(sorted_scattered_idxs).contiguous()
+    off = _i32(expert_offsets).contiguous()
+    E, H, I = w_proj_q.shape
+    L = ss.numel()
+    if act.shape != (L, I) or scale.shape != (E, H):
+        raise ValueError("shape mismatch")
+    o = torch.empty((L, H), dtype=act.dtype, device=act.device)
+    with _stage("down_fp8"):
+        check(_lib.load().mi_moe_down_fp8(_ptr(act), _ptr(w_proj_q), _ptr(scale), _ptr(o), _ptr(ss), _ptr(off), L, I, H,
+                                         E, _code(act.dtype), _stream()))
+    return o

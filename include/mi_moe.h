@@ -1,0 +1,158 @@
+/*
+ * mi_moe.h -- C ABI of the MI355X (gfx950) scattered-MoE forward kernels.
+ *
+ * One shared library (libmi_moe.so), plain C types only.  Every function
+ *   - takes device pointers the CALLER allocated (inputs, outputs and workspace); the library
+ *     never allocates, frees or keeps a pointer after it returns;
+ *   - validates its arguments on the host BEFORE anything is launched and returns
+ *       0  on success,
+ *      <0  an MI_MOE_E* argument / shape / alignment / dtype error (nothing was launched),
+ *      >0  the hipError_t of a failed launch;
+ *   - is asynchronous: work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ *     default stream); there is no host synchronisation and no device-to-host copy;
+ *   - is re-entrant and keeps no mutable global state.
+ *
+ * Index tensors are int32 inside the ABI.  Matrices are row-major and contiguous.  Expert weights
+ * are read in the module's native (E, out_features, in_features) layout, i.e. the contraction
+ * dimension is contiguous for both operands; no transposed copy is ever made.
+ *
+ * The reference reaches this path through a Python function boundary into the external
+ * `cute_kernels` package (lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:22-24); each entry
+ * point below names the reference call site it stands in for.
+ */
+#ifndef MI_MOE_H
+#define MI_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI_MOE_ABI_VERSION 1
+
+/* element types of activations / weights / logits */
+#define MI_MOE_F32 0
+#define MI_MOE_F16 1
+#define MI_MOE_BF16 2
+
+/* error codes (negative) */
+#define MI_MOE_OK 0
+#define MI_MOE_ENULL (-1)      /* a required pointer is NULL */
+#define MI_MOE_ESHAPE (-2)     /* a dimension is out of the supported range */
+#define MI_MOE_EDTYPE (-3)     /* unsupported element type for this entry point */
+#define MI_MOE_EALIGN (-4)     /* a pointer or leading dimension is not aligned as required */
+#define MI_MOE_EWORKSPACE (-5) /* workspace missing or too small */
+#define MI_MOE_EUNSUPPORTED (-6)
+
+typedef void* mi_moe_stream_t; /* hipStream_t */
+
+int mi_moe_abi_version(void);
+
+/* Human-readable text for a return code of any function below (static storage). */
+const char* mi_moe_strerror(int rc);
+
+/*
+ * Router top-k + softmax over the selected logits.
+ * Replaces: MoE._get_topk + F.softmax(...float()).type_as (moe.py:250-255, 338-344).
+ *   logits    (T, E) of `dtype`, 1 <= k <= E <= 1024
+ *   gates_out (T, k) of `dtype`  -- softmax in fp32 over the k selected values, rounded once
+ *   idx_out   (T, k) int32       -- experts in order (value descending, expert index ascending);
+ *                                   NaN orders as the largest value
+ */
+int mi_moe_router_topk_softmax(const void* logits, int T, int E, int k, int dtype,
+                               void* gates_out, int32_t* idx_out, mi_moe_stream_t stream);
+
+/*
+ * Fused router: logits = x @ gate_w^T rounded to `dtype` (+ optional per-expert fp32 bias, rounded
+ * again), then the top-k softmax above, in ONE pass over x.
+ * Replaces: MoE._compute_routing_weights (moe.py:246-257).
+ *   x (T, H), gate_w (E, H) of `dtype` (F16 / BF16), H % 8 == 0, E <= 64
+ *   bias       (E,) fp32 or NULL
+ *   logits_out (T, E) of `dtype` or NULL (only the training-time aux loss reads it)
+ */
+int mi_moe_router_fused(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,
+                        int dtype, void* logits_out, void* gates_out, int32_t* idx_out,
+                        mi_moe_stream_t stream);
+
+/*
+ * Histogram of expert ids.
+ * Replaces: continuous_count_cute / the bincount custom op (moe.py:27-44).
+ *   ids (L,) int32 with values in [0, E); counts_out (E,) uint32.  1 <= E <= 1024.
+ */
+int mi_moe_count(const int32_t* ids, int L, int E, uint32_t* counts_out, mi_moe_stream_t stream);
+
+/*
+ * Expert sort / bin: stable counting sort of the flat (T*k,) expert ids.
+ * Replaces: selected_experts.flatten().sort() + compute_bincount(...).cumsum(-1) (moe.py:263-271).
+ *   topk_idx          (T*k,) int32, values in [0, E)
+ *   sorted_expert     (T*k,) int32  non-decreasing expert ids
+ *   sorted_scattered  (T*k,) int32  flat slot id (t*k + j) of each sorted row; stable
+ *   expert_offsets    (E,)   int32  INCLUSIVE prefix sum of the per-expert counts
+ *   ws / ws_bytes     scratch of at least mi_moe_sort_bin_workspace_bytes(T*k, E) bytes, 16-byte aligned
+ */
+size_t mi_moe_sort_bin_workspace_bytes(int L, int E);
+int mi_moe_sort_bin(const int32_t* topk_idx, int T, int k, int E, int32_t* sorted_expert,
+                    int32_t* sorted_scattered, int32_t* expert_offsets, void* ws, size_t ws_bytes,
+                    mi_moe_stream_t stream);
+
+/*
+ * Grouped ("scatter2scatter") GEMM:  for every sorted row i with expert e_i
+ *     out[ orow(i), : ] = in[ irow(i), : ] @ w[e_i]^T
+ *   irow(i) = i                              if grouped_in   else sorted_scattered[i] / k
+ *   orow(i) = i                              if grouped_out  else sorted_scattered[i]
+ * Replaces: scattered_experts(...) without gates (moe.py:91-101).
+ *   in  (in_rows, K), w (E, N, K), out (L, N) of `dtype`; L = T*k rows in sorted order;
+ *   expert e owns sorted rows [expert_offsets[e-1], expert_offsets[e]).
+ */
+int mi_moe_scattered_gemm(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
+                          const int32_t* expert_offsets, int L, int K, int N, int E, int k,
+                          int grouped_in, int grouped_out, int dtype, mi_moe_stream_t stream);
+
+/* Same call with an explicit tile configuration (tuning / benchmarking): cfg = -1 picks one from the
+ * shape, 0 = 256x256 tile, 1 = 128x128, 2 = 32x256, 3 = one-thread-per-element fallback. */
+int mi_moe_scattered_gemm_cfg(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
+                              const int32_t* expert_offsets, int L, int K, int N, int E, int k,
+                              int grouped_in, int grouped_out, int dtype, int cfg, mi_moe_stream_t stream);
+
+/*
+ * Up-projection with SwiGLU fused into the epilogue:
+ *     h = x[sorted_scattered[i] / k] @ w_fc[e_i]^T  (2I wide: rows [0,I) of w_fc are "up", [I,2I) "gate")
+ *     act_out[i, :] = h[:I] * silu(h[I:])           (grouped order, `dtype`)
+ * Replaces: c_fc scattered_experts(grouped_out=True) + GLUActivation (moe.py:273-281, glu.py:42-43).
+ *   x (T, H), w_fc (E, 2I, H), act_out (L, I).
+ */
+int mi_moe_up_swiglu(const void* x, const void* w_fc, void* act_out, const int32_t* sorted_scattered,
+                     const int32_t* expert_offsets, int L, int H, int I, int E, int k, int dtype,
+                     mi_moe_stream_t stream);
+
+int mi_moe_up_swiglu_cfg(const void* x, const void* w_fc, void* act_out, const int32_t* sorted_scattered,
+                         const int32_t* expert_offsets, int L, int H, int I, int E, int k, int dtype, int cfg,
+                         mi_moe_stream_t stream);
+
+/*
+ * Gate-weighted combine:  y[t, :] = sum_j gates[t, j] * o[t*k + j, :]   (fp32 accumulation).
+ * Replaces: the gates contraction inside scattered_experts(gates=...) (moe.py:282-290).
+ *   o (T*k, H), gates (T, k), y (T, H) of `dtype`.
+ */
+int mi_moe_combine(const void* o, const void* gates, void* y, int T, int k, int H, int dtype,
+                   mi_moe_stream_t stream);
+
+/*
+ * Decode-shape variants with fp8 (OCP e4m3fn) expert weights and one fp32 scale per output channel.
+ * No counterpart in the reference (its fp8 support wraps nn.Linear only, lm_engine/fp8.py:63-73);
+ * semantics = dequantise (w * scale[:, None]) then the two calls above.
+ *   x / act / o are `dtype` (F16 / BF16); w_* are (E, out, in) bytes; *_scale are (E, out) fp32.
+ */
+int mi_moe_up_swiglu_fp8(const void* x, const void* w_fc_q, const float* w_fc_scale, void* act_out,
+                         const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int H, int I,
+                         int E, int k, int dtype, mi_moe_stream_t stream);
+int mi_moe_down_fp8(const void* act, const void* w_proj_q, const float* w_proj_scale, void* o_out,
+                    const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
+                    int E, int dtype, mi_moe_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_MOE_H */

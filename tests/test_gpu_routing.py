@@ -1,0 +1,129 @@
+"""GPU parity of the routing kernels against the CPU oracle (bit-exact indices, counts, order)."""
+
+import pytest
+import torch
+
+from oracle import moe_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from dolomite_engine_amd import ops
+
+    return ops
+
+
+def _logits(T, E, dtype, seed, ties=False):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, E, generator=g) * 0.7
+    if ties:  # coarse grid: many exact ties, including at the k / k+1 boundary
+        x = torch.round(x * 2) / 2
+    return x.to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k", [(1, 8, 2), (15, 8, 8), (512, 8, 2), (1000, 32, 8), (777, 40, 8), (64, 64, 6),
+                                   (33, 5, 1), (129, 100, 7), (65, 256, 9), (31, 1000, 64), (16, 1, 1)])
+@pytest.mark.parametrize("ties", [False, True])
+def test_topk_softmax(device, dtype, T, E, k, ties):
+    ops = _ops()
+    logits = _logits(T, E, dtype, seed=T * 131 + E * 7 + k, ties=ties)
+    print(f"topk T={T} E={E} k={k} {dtype} ties={ties}", flush=True)
+    gates, idx = ops.router_topk_softmax(logits.to(device), k)
+    vals, ref_idx = oracle.topk_canonical(logits, k)
+    ref_gates = oracle.softmax_topk(vals, dtype)
+    assert idx.dtype == torch.int32
+    assert torch.equal(idx.cpu().long(), ref_idx), "expert indices differ from the canonical top-k"
+    tol = {torch.float32: 2e-6, torch.bfloat16: 8e-3, torch.float16: 1e-3}[dtype]
+    torch.testing.assert_close(gates.cpu().float(), ref_gates.float(), rtol=tol, atol=tol * 0.1)
+    # at most one unit in the last place anywhere
+    if dtype != torch.float32:
+        ulp_diff = (gates.cpu().view(torch.int16).int() - ref_gates.view(torch.int16).int()).abs().max()
+        assert ulp_diff <= 1
+
+
+def test_topk_special_values(device):
+    ops = _ops()
+    x = torch.tensor([[0.0, -0.0, 1.0, float("-inf"), 1.0, float("inf"), -2.0, 0.5],
+                      [float("nan"), 1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0]])
+    gates, idx = ops.router_topk_softmax(x.to(device), 4)
+    assert idx[0].tolist() == [5, 2, 4, 7]
+    assert idx[1].tolist()[0] == 0  # NaN orders first, as in torch
+    _, ref = oracle.topk_canonical(x, 4)
+    assert torch.equal(idx.cpu().long(), ref)
+    # -0.0 and +0.0 tie: lower index first
+    y = torch.tensor([[-0.0, 0.0, -1.0, -1.0]])
+    _, idx = ops.router_topk_softmax(y.to(device), 2)
+    assert idx[0].tolist() == [0, 1]
+
+
+@pytest.mark.parametrize("T,k,E", [(0, 2, 8), (1, 1, 1), (15, 8, 8), (512, 2, 8), (64, 6, 64), (1024, 8, 32),
+                                   (1365, 6, 40), (16384, 8, 32), (32768, 8, 40), (5000, 3, 1000), (4099, 2, 3)])
+@pytest.mark.parametrize("skew", [False, True])
+def test_sort_bin(device, T, k, E, skew):
+    ops = _ops()
+    g = torch.Generator().manual_seed(T + 17 * k + E)
+    if skew:
+        p = torch.arange(1, E + 1, dtype=torch.float64).pow(-1.1)
+        sel = torch.multinomial(p.expand(max(T, 1), E), min(k, E), replacement=False, generator=g)[:T]
+        if k > E:
+            pytest.skip("k > E")
+    else:
+        sel = torch.rand(T, E, generator=g).argsort(dim=1)[:, :k]
+    sel = sel.reshape(T, k)
+    print(f"sort_bin T={T} k={k} E={E} skew={skew}", flush=True)
+    se, ss, off = ops.sort_bin(sel.to(device=device, dtype=torch.int32), E)
+    rse, rss, roff = oracle.sort_bin(sel, E)
+    assert torch.equal(off.cpu().long(), roff)
+    assert torch.equal(se.cpu().long(), rse)
+    assert torch.equal(ss.cpu().long(), rss)
+
+
+def test_sort_bin_all_one_expert(device):
+    ops = _ops()
+    T, k, E = 9000, 1, 16
+    sel = torch.full((T, k), 11, dtype=torch.int32)
+    se, ss, off = ops.sort_bin(sel.to(device), E)
+    assert torch.equal(ss.cpu().long(), torch.arange(T))
+    assert off.cpu().tolist() == [0] * 11 + [T] * 5
+    assert bool((se == 11).all())
+
+
+@pytest.mark.parametrize("L,E", [(0, 4), (1, 1), (1000, 8), (262144, 40), (100003, 1000)])
+def test_count(device, L, E):
+    ops = _ops()
+    g = torch.Generator().manual_seed(L + E)
+    ids = torch.randint(0, E, (L,), generator=g)
+    got = ops.continuous_count(ids.to(device), E)
+    assert got.dtype == torch.uint32
+    assert torch.equal(got.cpu().to(torch.int64), torch.bincount(ids, minlength=E))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E,k,bias", [(1, 64, 8, 2, False), (15, 32, 8, 8, False), (200, 256, 40, 8, True),
+                                          (1000, 1024, 32, 8, False), (64, 4096, 64, 6, False),
+                                          (333, 1536, 40, 8, True), (130, 48, 5, 1, False)])
+def test_router_fused(device, dtype, T, H, E, k, bias):
+    ops = _ops()
+    g = torch.Generator().manual_seed(T + H + E)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    w = (torch.randn(E, H, generator=g) * 0.02).to(dtype)
+    b = (torch.randn(E, generator=g) * 0.5) if bias else None
+    print(f"router_fused T={T} H={H} E={E} k={k} {dtype} bias={bias}", flush=True)
+    logits, gates, idx = ops.router_fused(x.to(device), w.to(device), k, bias=None if b is None else b.to(device),
+                                          return_logits=True)
+    logits = logits.cpu()
+    # (1) the logits are the oracle's up to one rounding step of the model dtype
+    ref_logits = oracle.router_logits(x, w, b)
+    torch.testing.assert_close(logits.float(), ref_logits.float(), rtol=1.6e-2 if dtype == torch.bfloat16 else 2e-3,
+                               atol=1e-3)
+    # (2) given the device's own logits, routing is bit-exact
+    vals, ref_idx = oracle.topk_canonical(logits, k)
+    assert torch.equal(idx.cpu().long(), ref_idx)
+    ref_gates = oracle.softmax_topk(vals, dtype)
+    ulp = (gates.cpu().view(torch.int16).int() - ref_gates.view(torch.int16).int()).abs().max()
+    assert ulp <= 1
+    # (3) without materialising the logits the result is the same
+    _, gates2, idx2 = ops.router_fused(x.to(device), w.to(device), k, bias=None if b is None else b.to(device))
+    assert torch.equal(idx2, idx) and torch.equal(gates2, gates)
