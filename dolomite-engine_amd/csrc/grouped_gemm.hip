@@ -55,8 +55,83 @@ struct GemmArgs {
   int remap;    // XCD-aware tile order
 };
 
-template <typename T, int BM, int BNW, int BK, int WM, int WN, bool GLU>
+
+// Tile -> (expert, row range, column tile).  Row tiles are numbered expert by expert (expert e has
+// ceil(n_e / BM) of them), column tiles innermost.  The walk over the E inclusive offsets is done by
+// one wavefront 64 experts at a time (one coalesced load + a shuffle scan) instead of E dependent
+// scalar loads; every wave of the workgroup does it redundantly, so no LDS or barrier is involved.
+// With `remap` the workgroup ids (dealt round-robin to the 8 XCDs) are permuted so that each XCD
+// owns a contiguous range of tiles.  Returns false for surplus workgroups.
+struct TileCoord {
+  int expert, row_begin, row_end, nt;
+};
+
+template <int BM>
+__device__ __forceinline__ bool decode_tile(const int32_t* __restrict__ off, int E, int n_tiles, int remap,
+                                            TileCoord& tc) {
+  const int lane = threadIdx.x & 63;
+  // pass 1: total number of row tiles
+  int total_m = 0;
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    const int e = e0 + lane;
+    const int end = e < E ? off[e] : 0;
+    const int prev = (e < E && e > 0) ? off[e - 1] : 0;
+    int t = e < E ? (end - prev + BM - 1) / BM : 0;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) t += __shfl_xor(t, o, 64);
+    total_m += t;
+  }
+  const int total = total_m * n_tiles;
+  int tile;
+  if (remap & 1) {
+    const int per = (total + 7) >> 3;
+    const int local = blockIdx.x >> 3;
+    if (local >= per) return false;
+    tile = (blockIdx.x & 7) * per + local;
+  } else {
+    tile = blockIdx.x;
+  }
+  if (tile >= total) return false;
+  const int mt = tile / n_tiles;
+  tc.nt = tile - mt * n_tiles;
+  // pass 2: the expert whose row tiles contain mt
+  int carry = 0;
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    const int e = e0 + lane;
+    const int end = e < E ? off[e] : 0;
+    const int prev = (e < E && e > 0) ? off[e - 1] : 0;
+    const int t = e < E ? (end - prev + BM - 1) / BM : 0;
+    int incl = t;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      int v = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += v;
+    }
+    incl += carry;
+    const uint64_t hit = __ballot(incl > mt);
+    if (hit) {
+      const int src = __ffsll((long long)hit) - 1;
+      const int first_tile = __shfl(incl - t, src, 64);
+      const int p = __shfl(prev, src, 64);
+      tc.expert = e0 + src;
+      tc.row_begin = p + (mt - first_tile) * BM;
+      tc.row_end = __shfl(end, src, 64);
+      return true;
+    }
+    carry = __shfl(incl, 63, 64);
+  }
+  return false;
+}
+
+// scheduling-group masks of __builtin_amdgcn_sched_group_barrier
+#define SG_MFMA 0x008
+#define SG_VMEM_RD 0x020
+#define SG_DS_RD 0x100
+#define SG_DS_WR 0x200
+
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool KTAIL>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
+  constexpr int BK = 64;
   constexpr int NT = WM * WN * 64;
   constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
   constexpr int RS = NT / CPR;              // tile rows covered by one pass of the workgroup
@@ -67,8 +142,13 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
   constexpr int WTN = BNW / WN;             // wave tile, weight rows
   constexpr int MB = WTM / 32, NB = WTN / 32;
   constexpr int STAGE_ELEMS = (BM + BNW) * BK;
-  static_assert(BK == 64 || BK == 32, "BK");
-  static_assert(RS % 8 == 0 && BM % RS == 0 && BNW % RS == 0, "tile/thread shape");
+  constexpr int NMFMA = MB * NB;            // MFMAs per 16-wide k step
+  constexpr int NRD = MB + NB;              // fragment reads per k step
+  constexpr int NWR = XCH + WCH;            // LDS chunk writes per K tile
+  constexpr int RD_PER = (NRD + NMFMA - 1) / NMFMA;
+  constexpr int WR_PER = (NWR + 2 * NMFMA - 1) / (2 * NMFMA);
+  constexpr int LD_PER = (NWR + NMFMA - 1) / NMFMA;
+  static_assert(RS % 16 == 0 && BM % RS == 0 && BNW % RS == 0, "tile/thread shape");
   static_assert(!GLU || NB % 2 == 0, "SwiGLU needs an even number of column blocks per wave");
   typedef typename Mfma32<T>::vec frag_t;
 
@@ -77,46 +157,10 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave % WM, wn = wave / WM;
-  const int32_t* __restrict__ off = a.expert_offsets;
 
-  // ---- which tile is mine --------------------------------------------------------------------
-  int total_m = 0;
-  {
-    int prev = 0;
-    for (int e = 0; e < a.E; ++e) {
-      int end = off[e];
-      total_m += (end - prev + BM - 1) / BM;
-      prev = end;
-    }
-  }
-  const int total = total_m * a.n_tiles;
-  int tile;
-  if (a.remap) {
-    const int per = (total + 7) >> 3;
-    const int local = blockIdx.x >> 3;
-    if (local >= per) return;
-    tile = (blockIdx.x & 7) * per + local;
-  } else {
-    tile = blockIdx.x;
-  }
-  if (tile >= total) return;
-  const int mt = tile / a.n_tiles, nt = tile - mt * a.n_tiles;
-  int expert = 0, row_begin = 0, row_end = 0;
-  {
-    int prev = 0, acc = 0;
-    for (int e = 0; e < a.E; ++e) {
-      int end = off[e];
-      int tiles = (end - prev + BM - 1) / BM;
-      if (mt < acc + tiles) {
-        expert = e;
-        row_begin = prev + (mt - acc) * BM;
-        row_end = end;
-        break;
-      }
-      acc += tiles;
-      prev = end;
-    }
-  }
+  TileCoord tc;
+  if (!decode_tile<BM>(a.expert_offsets, a.E, a.n_tiles, a.remap, tc)) return;
+  const int expert = tc.expert, row_begin = tc.row_begin, row_end = tc.row_end, nt = tc.nt;
 
   // ---- per-thread global sources ---------------------------------------------------------------
   const int c = tid % CPR;   // chunk within a tile row
@@ -147,8 +191,11 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
     woff[j] = (uint32_t)(half * a.N + col) * (uint32_t)a.K + c * 8;
   }
 
-  // swizzled LDS chunk slot of this thread's chunks (same for all its rows because RS % 8 == 0)
-  const int sw_c = (BK == 64) ? (c ^ (r0 & 7)) : (c ^ ((r0 >> 1) & 3));
+  // LDS tile layout: row r holds its eight 16-byte chunks at slots  chunk ^ swz(r),
+  // swz(r) = (r & 7) ^ ((r >> 3) & 1): any 8 consecutive rows AND any 16 consecutive rows of one
+  // logical chunk fall into distinct bank groups (row parity selects the upper / lower 32 banks).
+  // RS % 16 == 0, so all chunks of a thread share one swizzle.
+  const int sw_c = c ^ ((r0 & 7) ^ ((r0 >> 3) & 1));
   const int st_x = (r0 * CPR + sw_c) * 8;              // element offset inside the X tile
   const int st_w = BM * BK + (r0 * CPR + sw_c) * 8;    // ... inside the W tile (after the X tile)
 
@@ -156,35 +203,48 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
   const int nk = (a.K + BK - 1) / BK;
 
   auto load_global = [&](int kt) {
-    const int k0 = kt * BK;
-    const bool kvalid = (k0 + c * 8) < a.K;
+    int k0 = kt * BK;
+    if (KTAIL) {
+      // the last K tile may be partial: out-of-range chunks re-read chunk 0 of the row and are zeroed
+      const bool kvalid = (k0 + c * 8) < a.K;
+      const int koff = kvalid ? k0 : -(c * 8);
 #pragma unroll
-    for (int j = 0; j < XCH; ++j) {
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (kvalid) v = *reinterpret_cast<const u32x4*>(xbase + xoff[j] + k0);
-      xreg[j] = v;
-    }
+      for (int j = 0; j < XCH; ++j) {
+        u32x4 v = *reinterpret_cast<const u32x4*>(xbase + xoff[j] + koff);
+        xreg[j] = kvalid ? v : (u32x4){0u, 0u, 0u, 0u};
+      }
 #pragma unroll
-    for (int j = 0; j < WCH; ++j) {
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (kvalid) v = *reinterpret_cast<const u32x4*>(wbase + woff[j] + k0);
-      wreg[j] = v;
+      for (int j = 0; j < WCH; ++j) {
+        u32x4 v = *reinterpret_cast<const u32x4*>(wbase + woff[j] + koff);
+        wreg[j] = kvalid ? v : (u32x4){0u, 0u, 0u, 0u};
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < XCH; ++j) xreg[j] = *reinterpret_cast<const u32x4*>(xbase + xoff[j] + k0);
+#pragma unroll
+      for (int j = 0; j < WCH; ++j) wreg[j] = *reinterpret_cast<const u32x4*>(wbase + woff[j] + k0);
     }
   };
-  auto store_lds = [&](int stage) {
+  // chunk writes [first, first + count) of this thread's NWR chunks (X chunks first, then W chunks)
+  auto store_lds = [&](int stage, int first, int count) {
     T* s = smem + stage * STAGE_ELEMS;
 #pragma unroll
-    for (int j = 0; j < XCH; ++j) *reinterpret_cast<u32x4*>(s + st_x + j * RS * BK) = xreg[j];
-#pragma unroll
-    for (int j = 0; j < WCH; ++j) *reinterpret_cast<u32x4*>(s + st_w + j * RS * BK) = wreg[j];
+    for (int j = 0; j < NWR; ++j) {
+      if (j < first || j >= first + count) continue;
+      if (j < XCH)
+        *reinterpret_cast<u32x4*>(s + st_x + j * RS * BK) = xreg[j];
+      else
+        *reinterpret_cast<u32x4*>(s + st_w + (j - XCH) * RS * BK) = wreg[j - XCH];
+    }
   };
 
-  // ---- fragment read addresses ----------------------------------------------------------------------
+  // ---- fragment reads ---------------------------------------------------------------------------
   // lane l reads tile row (block_row0 + l%32), logical chunk 2*kk + l/32
   const int frow = lane & 31, fhalf = lane >> 5;
-  int frag_x_row[MB], frag_w_row[NB];
+  const int fswz = (frow & 7) ^ ((frow >> 3) & 1);  // block_row0 is a multiple of 32
+  int frag_x_off[MB], frag_w_off[NB];                // element offsets of the row inside a stage
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) frag_x_row[mb] = wm * WTM + mb * 32 + frow;
+  for (int mb = 0; mb < MB; ++mb) frag_x_off[mb] = (wm * WTM + mb * 32 + frow) * BK;
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     int r;
@@ -195,8 +255,22 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
     } else {
       r = wn * WTN + nb * 32 + frow;
     }
-    frag_w_row[nb] = r;
+    frag_w_off[nb] = BM * BK + r * BK;
   }
+  int chunk_off[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) chunk_off[kk] = ((kk * 2 + fhalf) ^ fswz) * 8;
+
+  frag_t xf[2][MB], wf[2][NB];
+  auto read_frags = [&](int stage, int kk, int buf) {
+    const T* s = smem + stage * STAGE_ELEMS + chunk_off[kk];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+      wf[buf][nb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_w_off[nb]));
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      xf[buf][mb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_x_off[mb]));
+  };
 
   f32x16 acc[NB][MB];
 #pragma unroll
@@ -206,39 +280,75 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[nb][mb][i] = 0.f;
 
+  auto mfma_step = [&](int buf) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = Mfma32<T>::run(wf[buf][nb], xf[buf][mb], acc[nb][mb]);
+  };
+
+  // ---- software pipeline ------------------------------------------------------------------------
+  // Per K tile (4 k-steps of 16), with LDS stages cur / nxt and fragment buffers 0 / 1:
+  //   step 0: MFMA(buf0) | read frags(step1, cur) -> buf1
+  //   step 1: MFMA(buf1) | read frags(step2, cur) -> buf0 | write first half of tile kt+1 -> nxt
+  //   step 2: MFMA(buf0) | read frags(step3, cur) -> buf1 | write second half            -> nxt
+  //   barrier            (nxt complete; everybody has fetched its last fragments of cur)
+  //   step 3: MFMA(buf1) | read frags(step0, nxt) -> buf0 | global loads of tile kt+2 -> registers
+  // The sched_group_barrier sequences ask the backend to issue the LDS / global instructions in the
+  // shadow of the MFMAs (one wave per SIMD: nothing else hides their issue slots).
   load_global(0);
-  store_lds(0);
+  store_lds(0, 0, NWR);
   __syncthreads();
+  load_global(nk > 1 ? 1 : 0);
+  read_frags(0, 0, 0);
 
+  // The last round stages a surplus tile (a re-read of the last one) that nobody consumes; keeping the
+  // loop body uniform keeps the accumulators in place (no peeled copy of the 256 accumulator registers).
   for (int kt = 0; kt < nk; ++kt) {
-    if (kt + 1 < nk) load_global(kt + 1);
-    const T* sx = smem + (kt & 1) * STAGE_ELEMS;
-    const T* sw = sx + BM * BK;
+    const int cur = kt & 1, nxt = cur ^ 1;
+    read_frags(cur, 1, 1);
+    mfma_step(0);
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      const int chunk = kk * 2 + fhalf;
-      frag_t xf[MB], wf[NB];
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        int r = frag_x_row[mb];
-        int pc = (BK == 64) ? (chunk ^ (r & 7)) : (chunk ^ ((r >> 1) & 3));
-        xf[mb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(sx + (r * CPR + pc) * 8));
-      }
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        int r = frag_w_row[nb];
-        int pc = (BK == 64) ? (chunk ^ (r & 7)) : (chunk ^ ((r >> 1) & 3));
-        wf[nb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(sw + (r * CPR + pc) * 8));
-      }
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = Mfma32<T>::run(wf[nb], xf[mb], acc[nb][mb]);
+    for (int i = 0; i < NMFMA; ++i) {
+      __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(SG_DS_RD, RD_PER, 0);
     }
-    if (kt + 1 < nk) store_lds((kt + 1) & 1);
-    __syncthreads();
-  }
+    __builtin_amdgcn_sched_barrier(0);
 
+    read_frags(cur, 2, 0);
+    store_lds(nxt, 0, NWR / 2);
+    mfma_step(1);
+#pragma unroll
+    for (int i = 0; i < NMFMA; ++i) {
+      __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(SG_DS_RD, RD_PER, 0);
+      __builtin_amdgcn_sched_group_barrier(SG_DS_WR, WR_PER, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    read_frags(cur, 3, 1);
+    store_lds(nxt, NWR / 2, NWR - NWR / 2);
+    mfma_step(0);
+#pragma unroll
+    for (int i = 0; i < NMFMA; ++i) {
+      __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(SG_DS_RD, RD_PER, 0);
+      __builtin_amdgcn_sched_group_barrier(SG_DS_WR, WR_PER, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+
+    read_frags(nxt, 0, 0);
+    load_global(kt + 2 < nk ? kt + 2 : nk - 1);  // the surplus load of the last round is never used
+    mfma_step(1);
+#pragma unroll
+    for (int i = 0; i < NMFMA; ++i) {
+      __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(SG_DS_RD, RD_PER, 0);
+      __builtin_amdgcn_sched_group_barrier(SG_VMEM_RD, LD_PER, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
   // ---- epilogue ---------------------------------------------------------------------------------
   // acc[nb][mb][i]: weight row (output column) = 8*(i/4) + 4*(lane/32) + i%4 of block nb,
   //                 activation row             = lane%32 of block mb
@@ -275,6 +385,582 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Main kernel: global -> LDS by DMA (global_load_lds_dwordx4), 4 LDS stages of 32 k each.
+//
+// The register-staged kernel above keeps only one K tile in flight; under load the L2 -> CU latency
+// exceeds one tile's worth of MFMA time and the matrix cores idle.  Here the tiles never pass through
+// VGPRs: every wave issues 16-byte-per-lane DMA loads whose destination is a contiguous 1 KiB run of
+// LDS (lane i -> base + 16*i).  Three tiles are in flight while a fourth is consumed.
+//
+//   stage layout   (BM + BNW) rows x 32 k, 64 bytes per row = 4 slots of 16 bytes;
+//                  slot of logical chunk c in row r:  c ^ ((r >> 2) & 3)   (ds_read_b128 conflict-free)
+//   DMA mapping    one wave instruction fills 16 rows: lane l -> row l/4, slot l%4, so the lane fetches
+//                  logical chunk (l%4) ^ ((row >> 2) & 3) of its row: the swizzle is applied on the
+//                  global side, 4 lanes still cover one contiguous 64-byte piece of a row
+//   iteration kt   (stage cur = kt % 4, fragment buffers 0/1, two k-steps of 16)
+//       A: MFMA(step 0, buf0)      | ds_read step 1 of cur -> buf1
+//       s_waitcnt vmcnt(2 tiles)   : my share of tile kt+1 has landed;  lgkmcnt(0): my reads of cur are done
+//       s_barrier                  : tile kt+1 complete, stage cur free
+//       B: MFMA(step 1, buf1)      | ds_read step 0 of tile kt+1 -> buf0 | DMA tile kt+4 -> stage cur
+// The waits are explicit (s_waitcnt immediates); a fence-carrying __syncthreads would drain all DMA.
+// ------------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ constexpr int waitcnt_imm(int vm, int lgkm) {
+  // gfx9 encoding: vmcnt = {imm[15:14], imm[3:0]}, expcnt = imm[6:4] (7 = no wait), lgkmcnt = imm[11:8]
+  return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8);
+}
+
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU>
+__global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GemmArgs a) {
+  constexpr int BK = 32;
+  constexpr int NSTAGE = 4;
+  constexpr int NW = WM * WN;
+  constexpr int NT = NW * 64;
+  constexpr int ROWS = BM + BNW;
+  constexpr int STAGE_BYTES = ROWS * BK * 2;
+  constexpr int NLD = ROWS / 16 / NW;       // DMA instructions per wave per tile
+  constexpr int BN = GLU ? BNW / 2 : BNW;
+  constexpr int WTM = BM / WM, WTN = BNW / WN;
+  constexpr int MB = WTM / 32, NB = WTN / 32;
+  constexpr int NMFMA = MB * NB;
+  constexpr int NRD = MB + NB;
+  constexpr int RD_PER = (NRD + NMFMA - 1) / NMFMA;
+  constexpr int LD_PER = (NLD + NMFMA - 1) / NMFMA;
+  static_assert(ROWS % (16 * NW) == 0 && BM % 16 == 0, "tile/wave shape");
+  static_assert(!GLU || NB % 2 == 0, "SwiGLU needs an even number of column blocks per wave");
+  static_assert(3 * NLD <= 63, "vmcnt range");
+  typedef typename Mfma32<T>::vec frag_t;
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  typedef const __attribute__((address_space(1))) void* glb_ptr_t;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % WM, wn = wave / WM;
+
+  TileCoord tc;
+  if (!decode_tile<BM>(a.expert_offsets, a.E, a.n_tiles, a.remap, tc)) return;
+  const int expert = tc.expert, row_begin = tc.row_begin, row_end = tc.row_end, nt = tc.nt;
+
+  // ---- DMA sources: instruction j of this wave fills stage rows [(j*NW + wave)*16, +16) -----------
+  constexpr int WROWS_MUL = GLU ? 2 : 1;
+  const T* __restrict__ xbase = static_cast<const T*>(a.in);
+  const T* __restrict__ wbase = static_cast<const T*>(a.w) + (size_t)expert * WROWS_MUL * a.N * a.K;
+  const int lchunk = (lane & 3) ^ ((lane >> 4) & 3);  // (row >> 2) & 3 == (lane >> 4) & 3: groups are 16-row aligned
+  const T* src[NLD];
+#pragma unroll
+  for (int j = 0; j < NLD; ++j) {
+    const int r = (j * NW + wave) * 16 + (lane >> 2);  // stage row
+    if (r < BM) {
+      int srow = row_begin + r;
+      if (srow > row_end - 1) srow = row_end - 1;  // tail rows re-read the last valid row; never stored
+      const int s = a.gather ? a.sorted_scattered[srow] / a.kdiv : srow;
+      src[j] = xbase + (size_t)s * a.K + lchunk * 8;
+    } else {
+      const int wr = r - BM;
+      int col, half = 0;
+      if (GLU) {
+        half = wr >= BN;
+        col = nt * BN + (half ? wr - BN : wr);
+      } else {
+        col = nt * BN + wr;
+      }
+      if (col > a.N - 1) col = a.N - 1;  // column tail re-reads the last weight row; never stored
+      src[j] = wbase + ((size_t)half * a.N + col) * a.K + lchunk * 8;
+    }
+  }
+  const int nk = a.K / BK;
+  auto dma_tile = [&](int kt, int stage) {
+    const int k0 = (kt < nk ? kt : nk - 1) * BK;  // surplus rounds re-fetch the last tile; never consumed
+#pragma unroll
+    for (int j = 0; j < NLD; ++j) {
+      unsigned char* dst = smem_raw + stage * STAGE_BYTES + (j * NW + wave) * 1024;
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)(src[j] + k0), (lds_ptr_t)dst, 16, 0, 0);
+    }
+  };
+
+  // ---- fragment reads --------------------------------------------------------------------------------
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int fswz = (frow >> 2) & 3;  // block rows start at multiples of 32
+  int frag_x_off[MB], frag_w_off[NB];  // byte offset of the fragment row inside a stage
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) frag_x_off[mb] = (wm * WTM + mb * 32 + frow) * (BK * 2);
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    int r;
+    if (GLU) {
+      constexpr int HB = NB / 2;
+      int h = nb >= HB;
+      r = h * BN + wn * (WTN / 2) + (h ? nb - HB : nb) * 32 + frow;
+    } else {
+      r = wn * WTN + nb * 32 + frow;
+    }
+    frag_w_off[nb] = (BM + r) * (BK * 2);
+  }
+  const int chunk_byte[2] = {((0 + fhalf) ^ fswz) * 16, ((2 + fhalf) ^ fswz) * 16};
+
+  frag_t xf[2][MB], wf[2][NB];
+  auto read_frags = [&](int stage, int kk, int buf) {
+    const unsigned char* s = smem_raw + stage * STAGE_BYTES + chunk_byte[kk];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+      wf[buf][nb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_w_off[nb]));
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      xf[buf][mb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_x_off[mb]));
+  };
+
+  f32x16 acc[NB][MB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[nb][mb][i] = 0.f;
+
+  auto mfma_step = [&](int buf) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = Mfma32<T>::run(wf[buf][nb], xf[buf][mb], acc[nb][mb]);
+  };
+
+  // ---- pipeline ----------------------------------------------------------------------------------------
+  dma_tile(0, 0);
+  dma_tile(1, 1);
+  dma_tile(2, 2);
+  dma_tile(3, 3);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(3 * NLD, 0));
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  read_frags(0, 0, 0);
+
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & (NSTAGE - 1), nxt = (kt + 1) & (NSTAGE - 1);
+    read_frags(cur, 1, 1);
+    mfma_step(0);
+#pragma unroll
+    for (int i = 0; i < NMFMA; ++i) {
+      __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(SG_DS_RD, RD_PER, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * NLD, 0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+
+    read_frags(nxt, 0, 0);
+    dma_tile(kt + 4, cur);
+    mfma_step(1);
+#pragma unroll
+    for (int i = 0; i < NMFMA; ++i) {
+      __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(SG_DS_RD, RD_PER, 0);
+      __builtin_amdgcn_sched_group_barrier(SG_VMEM_RD, LD_PER, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));  // surplus DMA must not outlive the workgroup's LDS
+
+  // ---- epilogue ---------------------------------------------------------------------------------
+  T* __restrict__ out = static_cast<T*>(a.out);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int row = row_begin + wm * WTM + mb * 32 + frow;
+    if (row >= row_end) continue;
+    const int orow = a.scatter ? a.sorted_scattered[row] : row;
+    T* orow_ptr = out + (size_t)orow * a.N;
+    constexpr int OB = GLU ? NB / 2 : NB;
+#pragma unroll
+    for (int nb = 0; nb < OB; ++nb) {
+      const int col0 = nt * BN + (GLU ? wn * (WTN / 2) : wn * WTN) + nb * 32 + fhalf * 4;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int col = col0 + g * 8;
+        if (col >= a.N) continue;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (GLU) {
+            float up = acc[nb][mb][g * 4 + i];
+            float gt = acc[nb + NB / 2][mb][g * 4 + i];
+            v[i] = up * silu_f32(gt);
+          } else {
+            v[i] = acc[nb][mb][g * 4 + i];
+          }
+        }
+        u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+        *reinterpret_cast<u32x2*>(orow_ptr + col) = p;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Persistent variant of the DMA kernel: one workgroup per CU walks a list of tiles and the 4-stage
+// LDS ring runs straight through the tile boundaries.
+//
+// A workgroup that handles one tile pays, per tile, for a launch, the tile lookup, the row-index
+// loads, an empty pipeline (three stages of DMA latency) and an epilogue during which nothing is in
+// flight; with K = 1536 that is as long as the MFMA work itself.  Here
+//   * the DMA for the first four K slices of tile i+1 is issued during the last four slices of tile i,
+//   * the lookup of tile i+2 comes from a per-expert table in LDS (no global loads) and its row-index
+//     loads are issued before the epilogue of tile i and consumed after it,
+//   * the epilogue stages each 32 x 64 block of results through a per-wave LDS scratch so that global
+//     stores are 16 bytes per lane and 128 contiguous bytes per row.
+// Tile order: workgroup b serves XCD b % 8 (hardware deals workgroup ids round-robin to the XCDs); the
+// XCD's contiguous tile range is dealt to its workgroups in turn, so at any moment the CUs of one XCD
+// work on neighbouring tiles (same expert weights, shared activation rows) out of one L2.
+// ------------------------------------------------------------------------------------------------
+
+#define PERSIST_MAX_E 256
+
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool SCHED>
+__global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(GemmArgs a) {
+  static_assert(BK == 32 || BK == 64, "BK");
+  constexpr int NSTAGE = BK == 32 ? 4 : 2;   // ring of 128 KiB either way
+  constexpr int STEPS = BK / 16;             // MFMA k-steps per ring stage
+  constexpr int RPI = BK == 32 ? 16 : 8;     // stage rows filled by one DMA instruction (1 KiB)
+  constexpr int LROW_SHIFT = BK == 32 ? 2 : 3;  // lane -> row within the instruction's rows
+  constexpr int NW = WM * WN;
+  constexpr int ROWS = BM + BNW;
+  constexpr int STAGE_BYTES = ROWS * BK * 2;
+  constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
+  constexpr int EPI_COLS = NW > 4 ? 32 : 64; // per-wave epilogue scratch: 32 rows x EPI_COLS columns
+  constexpr int EPI_BYTES = 32 * EPI_COLS * 2;
+  constexpr int EPI_OB = EPI_COLS / 32;      // 32-column blocks per epilogue pass
+  constexpr int EPI_CPR = EPI_COLS / 8;      // 16-byte chunks per scratch row
+  constexpr int NLD = ROWS / RPI / NW;       // DMA instructions per wave per K slice
+  constexpr int NXLD = BM / RPI / NW;        // ... of which activation rows (the first NXLD)
+  constexpr int BN = GLU ? BNW / 2 : BNW;
+  constexpr int WTM = BM / WM, WTN = BNW / WN;
+  constexpr int MB = WTM / 32, NB = WTN / 32;
+  constexpr int OB = GLU ? NB / 2 : NB;      // output column blocks per wave
+  constexpr int NMFMA = MB * NB;
+  constexpr int NRD = MB + NB;
+  constexpr int RD_PER = (NRD + NMFMA - 1) / NMFMA;
+  constexpr int LD_PER = (NLD + NMFMA - 1) / NMFMA;
+  static_assert(BM % (16 * NW) == 0 && BNW % (16 * NW) == 0 && NW % 2 == 0, "tile/wave shape");
+  static_assert(OB % EPI_OB == 0, "epilogue pass shape");
+  static_assert((NSTAGE - 1) * NLD <= 63, "vmcnt range");
+  typedef typename Mfma32<T>::vec frag_t;
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  typedef const __attribute__((address_space(1))) void* glb_ptr_t;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  // [ring: 4 stages][epilogue scratch: NW x 4 KiB][expert table: E x (tiles inclusive, row end)]
+  int* etab = reinterpret_cast<int*>(smem_raw + RING_BYTES + NW * EPI_BYTES);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % WM, wn = wave / WM;
+
+  // ---- per-expert table: etab[2e] = row tiles of experts 0..e, etab[2e+1] = offsets[e] ---------------
+  if (wave == 0) {
+    int carry = 0;
+    for (int e0 = 0; e0 < a.E; e0 += 64) {
+      const int e = e0 + lane;
+      const int end = e < a.E ? a.expert_offsets[e] : 0;
+      const int prev = (e < a.E && e > 0) ? a.expert_offsets[e - 1] : 0;
+      const int t = e < a.E ? (end - prev + BM - 1) / BM : 0;
+      int incl = t;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        int v = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += v;
+      }
+      incl += carry;
+      if (e < a.E) {
+        etab[2 * e] = incl;
+        etab[2 * e + 1] = end;
+      }
+      carry = __shfl(incl, 63, 64);
+    }
+  }
+  __syncthreads();
+  const int total = etab[2 * (a.E - 1)] * a.n_tiles;
+  const int per = (total + 7) >> 3;
+  const int xcd = blockIdx.x & 7, slot0 = blockIdx.x >> 3, nslot = gridDim.x >> 3;
+
+  // i-th tile of this workgroup, or -1
+  auto tile_of = [&](int i) -> int {
+    const int local = slot0 + i * nslot;
+    const int t = xcd * per + local;
+    return (local < per && t < total) ? t : -1;
+  };
+  // tile id -> coordinates, from the LDS table (wave-uniform result)
+  auto locate = [&](int tile, TileCoord& tc) {
+    const int mt = tile / a.n_tiles;
+    tc.nt = tile - mt * a.n_tiles;
+    for (int e0 = 0; e0 < a.E; e0 += 64) {
+      const int e = e0 + lane;
+      const int incl = e < a.E ? etab[2 * e] : 0x7fffffff;
+      const uint64_t hit = __ballot(incl > mt);
+      if (hit) {
+        const int ex = e0 + __ffsll((long long)hit) - 1;
+        const int first_tile = ex > 0 ? etab[2 * (ex - 1)] : 0;
+        const int prev = ex > 0 ? etab[2 * (ex - 1) + 1] : 0;
+        tc.expert = ex;
+        tc.row_begin = prev + (mt - first_tile) * BM;
+        tc.row_end = etab[2 * ex + 1];
+        return;
+      }
+    }
+    tc.expert = 0; tc.row_begin = 0; tc.row_end = 1;  // unreachable for a valid tile id
+  };
+
+  // ---- DMA sources -----------------------------------------------------------------------------------
+  // A tile's sources are NLD 32-bit byte offsets per lane (activation rows relative to the input
+  // matrix, weight rows relative to the expert's weight matrix) plus the expert's scalar base; the K
+  // position is added on the scalar side, so a DMA instruction is "scalar base + lane offset".
+  constexpr int WROWS_MUL = GLU ? 2 : 1;
+  const unsigned char* __restrict__ xbase = static_cast<const unsigned char*>(a.in);
+  const unsigned char* __restrict__ wall = static_cast<const unsigned char*>(a.w);
+  const size_t expert_bytes = (size_t)WROWS_MUL * a.N * a.K * sizeof(T);
+  // logical 16-byte chunk this lane fetches so that it lands in its swizzled slot (see read_frags):
+  //   BK = 32: row = 16*grp + lane/4, slot = lane%4, swizzle (row >> 2) & 3
+  //   BK = 64: row =  8*grp + lane/8, slot = lane%8, swizzle (row & 7) ^ ((row >> 3) & 1); grp parity == wave parity
+  const int lchunk = BK == 32 ? ((lane & 3) ^ ((lane >> 4) & 3)) : ((lane & 7) ^ (lane >> 3) ^ (wave & 1));
+  struct TileSrc {
+    uint32_t off[NLD];
+    const unsigned char* wbase;
+  };
+  // sorted-order row of the activation rows this lane fetches (clamped into the tile's expert)
+  auto load_rows = [&](const TileCoord& tc, int (&raw)[NXLD]) {
+#pragma unroll
+    for (int j = 0; j < NXLD; ++j) {
+      int srow = tc.row_begin + (j * NW + wave) * RPI + (lane >> LROW_SHIFT);
+      if (srow > tc.row_end - 1) srow = tc.row_end - 1;  // tail rows re-read the last valid row; never stored
+      raw[j] = a.gather ? a.sorted_scattered[srow] : srow;
+    }
+  };
+  auto make_src = [&](const TileCoord& tc, const int (&raw)[NXLD], TileSrc& ts) {
+    ts.wbase = wall + (size_t)tc.expert * expert_bytes;
+#pragma unroll
+    for (int j = 0; j < NLD; ++j) {
+      if (j < NXLD) {
+        const int s = a.gather ? raw[j] / a.kdiv : raw[j];
+        ts.off[j] = ((uint32_t)s * (uint32_t)a.K + lchunk * 8) * (uint32_t)sizeof(T);
+      } else {
+        const int wr = ((j - NXLD) * NW + wave) * RPI + (lane >> LROW_SHIFT);
+        int col, half = 0;
+        if (GLU) {
+          half = wr >= BN;
+          col = tc.nt * BN + (half ? wr - BN : wr);
+        } else {
+          col = tc.nt * BN + wr;
+        }
+        if (col > a.N - 1) col = a.N - 1;  // column tail re-reads the last weight row; never stored
+        ts.off[j] = ((uint32_t)(half * a.N + col) * (uint32_t)a.K + lchunk * 8) * (uint32_t)sizeof(T);
+      }
+    }
+  };
+  // slice kt of tile `cur`, or (from_next) of tile `next`, into ring stage `stage`
+  auto dma_slice = [&](const TileSrc& cur, const TileSrc& next, bool from_next, int kt, int stage) {
+    const size_t kbytes = (size_t)kt * BK * sizeof(T);
+    const unsigned char* xs = xbase + kbytes;
+    const unsigned char* ws = (from_next ? next.wbase : cur.wbase) + kbytes;
+#pragma unroll
+    for (int j = 0; j < NLD; ++j) {
+      // activation rows fill stage rows [0, BM), weight rows [BM, BM + BNW)
+      const int grp = j < NXLD ? (j * NW + wave) : (BM / RPI + (j - NXLD) * NW + wave);
+      unsigned char* dst = smem_raw + stage * STAGE_BYTES + grp * 1024;
+      const uint32_t o = from_next ? next.off[j] : cur.off[j];
+      __builtin_amdgcn_global_load_lds((glb_ptr_t)((j < NXLD ? xs : ws) + o), (lds_ptr_t)dst, 16, 0, 0);
+    }
+  };
+
+  // ---- fragment reads ----------------------------------------------------------------------------------
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int fswz = BK == 32 ? ((frow >> 2) & 3) : ((frow & 7) ^ ((frow >> 3) & 1));
+  int frag_x_off[MB], frag_w_off[NB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) frag_x_off[mb] = (wm * WTM + mb * 32 + frow) * (BK * 2);
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    int r;
+    if (GLU) {
+      constexpr int HB = NB / 2;
+      int h = nb >= HB;
+      r = h * BN + wn * (WTN / 2) + (h ? nb - HB : nb) * 32 + frow;
+    } else {
+      r = wn * WTN + nb * 32 + frow;
+    }
+    frag_w_off[nb] = (BM + r) * (BK * 2);
+  }
+  int chunk_byte[STEPS];
+#pragma unroll
+  for (int kk = 0; kk < STEPS; ++kk) chunk_byte[kk] = ((2 * kk + fhalf) ^ fswz) * 16;
+
+  frag_t xf[2][MB], wf[2][NB];
+  auto read_frags = [&](int stage, int kk, int buf) {
+    const unsigned char* s = smem_raw + stage * STAGE_BYTES + chunk_byte[kk];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+      wf[buf][nb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_w_off[nb]));
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      xf[buf][mb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_x_off[mb]));
+  };
+
+  f32x16 acc[NB][MB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[nb][mb][i] = 0.f;
+
+  auto mfma_step = [&](int buf) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = Mfma32<T>::run(wf[buf][nb], xf[buf][mb], acc[nb][mb]);
+  };
+
+  int g = 0;  // running K-slice count; slice g lives in ring stage g % NSTAGE
+  // one K slice: consume stage g % NSTAGE, then refill it with slice `kload` of tile cur / next
+  auto slice = [&](const TileSrc& tcur, const TileSrc& tnext, bool from_next, int kload) {
+    const int cur = g & (NSTAGE - 1), nxt = (g + 1) & (NSTAGE - 1);
+#pragma unroll
+    for (int st = 0; st < STEPS - 1; ++st) {
+      read_frags(cur, st + 1, (st + 1) & 1);
+      mfma_step(st & 1);
+      if (SCHED) {
+#pragma unroll
+        for (int i = 0; i < NMFMA; ++i) {
+          __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(SG_DS_RD, RD_PER, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm((NSTAGE - 2) * NLD, 0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(nxt, 0, 0);
+    dma_slice(tcur, tnext, from_next, kload, cur);
+    mfma_step((STEPS - 1) & 1);
+    if (SCHED) {
+#pragma unroll
+      for (int i = 0; i < NMFMA; ++i) {
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_RD, RD_PER, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_VMEM_RD, LD_PER, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    ++g;
+  };
+
+  // ---- epilogue of one tile: acc -> (SwiGLU) -> LDS scratch -> 16-byte row-contiguous stores -----------
+  T* __restrict__ out = static_cast<T*>(a.out);
+  unsigned char* scratch = smem_raw + RING_BYTES + wave * EPI_BYTES;
+  auto epilogue = [&](const TileCoord& tc) {
+    // scratch row r keeps its EPI_CPR 16-byte chunks at slots chunk ^ swz(r): the 8-byte writes of a
+    // wave (32 rows, one chunk) and the 16-byte read-back both spread over all banks
+    auto swz = [](int r) { return EPI_CPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3); };
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+      for (int og = 0; og < OB / EPI_OB; ++og) {
+        // write the 32 x EPI_COLS block: lane holds row frow, columns ob*32 + g*8 + fhalf*4 + [0,4)
+#pragma unroll
+        for (int ob = 0; ob < EPI_OB; ++ob) {
+          const int nb = og * EPI_OB + ob;
+#pragma unroll
+          for (int gq = 0; gq < 4; ++gq) {
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              if (GLU) {
+                const float up = acc[nb][mb][gq * 4 + i];
+                const float gt = acc[nb + NB / 2][mb][gq * 4 + i];
+                v[i] = up * gt * __builtin_amdgcn_rcpf(1.0f + __expf(-gt));
+              } else {
+                v[i] = acc[nb][mb][gq * 4 + i];
+              }
+            }
+            const int chunk = ob * 4 + gq;
+            const u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+            *reinterpret_cast<u32x2*>(scratch + frow * (EPI_COLS * 2) + ((chunk ^ swz(frow)) * 16) + fhalf * 8) = p;
+          }
+        }
+        // read back: lane -> row it*RPP + lane/EPI_CPR, 16-byte chunk lane%EPI_CPR
+        constexpr int RPP = 64 / EPI_CPR;  // rows per read-back pass
+        const int cchunk = lane % EPI_CPR;
+        const int col = tc.nt * BN + (GLU ? wn * (WTN / 2) : wn * WTN) + og * EPI_COLS + cchunk * 8;
+#pragma unroll
+        for (int it = 0; it < 32 / RPP; ++it) {
+          const int r = it * RPP + lane / EPI_CPR;
+          const u32x4 val = *reinterpret_cast<const u32x4*>(scratch + r * (EPI_COLS * 2) + ((cchunk ^ swz(r)) * 16));
+          const int row = tc.row_begin + wm * WTM + mb * 32 + r;
+          if (row < tc.row_end && col < a.N) {
+            const int orow = a.scatter ? a.sorted_scattered[row] : row;
+            *reinterpret_cast<u32x4*>(out + (size_t)orow * a.N + col) = val;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[nb][mb][i] = 0.f;
+  };
+
+  // ---- tile loop -------------------------------------------------------------------------------------------
+  const int nk = a.K / BK;  // >= NSTAGE (host-checked)
+  int t0 = tile_of(0);
+  if (t0 < 0) return;
+  TileCoord c0, c1;
+  locate(t0, c0);
+  int t1 = tile_of(1);
+  if (t1 >= 0) locate(t1, c1); else c1 = c0;
+  TileSrc src_cur, src_next;
+  {
+    int raw0[NXLD], raw1[NXLD];
+    load_rows(c0, raw0);
+    load_rows(c1, raw1);
+    make_src(c0, raw0, src_cur);
+    make_src(c1, raw1, src_next);
+  }
+#pragma unroll
+  for (int st = 0; st < NSTAGE; ++st) dma_slice(src_cur, src_cur, false, st, st);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm((NSTAGE - 1) * NLD, 0));
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  read_frags(0, 0, 0);
+
+  for (int i = 0;; ++i) {
+    // the ring runs on into the next tile: the last NSTAGE slices refill with its first NSTAGE
+    for (int kt = 0; kt < nk; ++kt) {
+      const bool from_next = kt >= nk - NSTAGE;
+      slice(src_cur, src_next, from_next, from_next ? kt + NSTAGE - nk : kt + NSTAGE);
+    }
+    const int t2 = tile_of(i + 2);
+    TileCoord c2 = c1;
+    if (t2 >= 0) locate(t2, c2);
+    int raw2[NXLD];
+    load_rows(c2, raw2);
+    epilogue(c0);
+    if (t1 < 0) break;
+    c0 = c1;
+    c1 = c2;
+    t1 = t2;
+    src_cur = src_next;
+    make_src(c2, raw2, src_next);
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));  // surplus DMA must not outlive the workgroup's LDS
+}
+
 // ---- any-shape / any-dtype fallback (one thread per output element) ------------------------------
 // Used for fp32 and for shapes the tiled kernel does not take (K % 8 != 0, N % 4 != 0, unaligned
 // pointers).  Correct, not fast.
@@ -301,11 +987,11 @@ __global__ __launch_bounds__(256) void grouped_gemm_naive_kernel(GemmArgs a) {
 
 // ---- host side ------------------------------------------------------------------------------------
 
-template <typename T, int BM, int BNW, int BK, int WM, int WN, bool GLU>
-static int launch_tiled(GemmArgs a, hipStream_t s) {
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool KTAIL>
+static int launch_tiled_k(GemmArgs a, hipStream_t s) {
   constexpr int BN = GLU ? BNW / 2 : BNW;
-  constexpr size_t lds = 2ull * (BM + BNW) * BK * sizeof(T);
-  auto kern = grouped_gemm_kernel<T, BM, BNW, BK, WM, WN, GLU>;
+  constexpr size_t lds = 2ull * (BM + BNW) * 64 * sizeof(T);
+  auto kern = grouped_gemm_kernel<T, BM, BNW, WM, WN, GLU, KTAIL>;
   if (lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -320,6 +1006,55 @@ static int launch_tiled(GemmArgs a, hipStream_t s) {
   return mi_launch_status();
 }
 
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU>
+static int launch_tiled(GemmArgs a, hipStream_t s) {
+  if (a.K % 64 == 0) return launch_tiled_k<T, BM, BNW, WM, WN, GLU, false>(a, s);
+  return launch_tiled_k<T, BM, BNW, WM, WN, GLU, true>(a, s);
+}
+
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU>
+static int launch_dma(GemmArgs a, hipStream_t s) {
+  constexpr int BN = GLU ? BNW / 2 : BNW;
+  constexpr size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T);
+  auto kern = grouped_gemm_dma_kernel<T, BM, BNW, WM, WN, GLU>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
+  a.n_tiles = mi_ceil_div(a.N, BN);
+  long max_m = (long)a.L / BM + (a.E < a.L ? a.E : a.L);
+  long grid = max_m * a.n_tiles;
+  grid = (grid + 7) / 8 * 8;
+  if (grid > 0x7fffffffL) return MI_MOE_ESHAPE;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WM * WN * 64), lds, s, a);
+  return mi_launch_status();
+}
+
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool SCHED>
+static int launch_persistent(GemmArgs a, hipStream_t s) {
+  constexpr int BN = GLU ? BNW / 2 : BNW;
+  constexpr int NW = WM * WN;
+  const size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T) + (size_t)NW * (NW > 4 ? 2048 : 4096) + (size_t)a.E * 8;
+  auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, BK, SCHED>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return (int)e;
+  a.n_tiles = mi_ceil_div(a.N, BN);
+  int dev = 0, cus = 0;
+  if ((e = hipGetDevice(&dev)) != hipSuccess) return (int)e;
+  if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return (int)e;
+  long max_tiles = ((long)a.L / BM + (a.E < a.L ? a.E : a.L)) * a.n_tiles;
+  long grid = cus < max_tiles ? cus : max_tiles;
+  grid = (grid + 7) / 8 * 8;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, a);
+  return mi_launch_status();
+}
+
+static bool persistent_ok(const GemmArgs& a) {
+  return a.K % 32 == 0 && a.K >= 128 && a.N % 8 == 0 && a.E <= PERSIST_MAX_E && mi_aligned(a.out, 16);
+}
+
 template <typename T, bool GLU>
 static int launch_naive(GemmArgs a, hipStream_t s) {
   dim3 grid(mi_ceil_div(a.L, 4), mi_ceil_div(a.N, 64));
@@ -328,13 +1063,22 @@ static int launch_naive(GemmArgs a, hipStream_t s) {
   return mi_launch_status();
 }
 
-// tile configurations: 0 = 256x256 (4 waves), 1 = 128x128 (4 waves), 2 = 32x128 (4 waves), 3 = naive
+// tile configurations
+//   0 / 1 / 2  register-staged 256x256 / 128x128 / 32x256 (any K % 8 == 0)
+//   3          one thread per output element (any shape, any dtype)
+//   4          DMA-staged 128x128, one tile per workgroup (K % 32 == 0)
+//   5 / 6      persistent DMA-staged 256x256, 8 waves, 32-wide / 64-wide K slices
 template <typename T, bool GLU>
 static int dispatch_cfg(GemmArgs a, int cfg, hipStream_t s) {
   switch (cfg) {
-    case 0: return launch_tiled<T, 256, 256, 64, 2, 2, GLU>(a, s);
-    case 1: return launch_tiled<T, 128, 128, 64, 2, 2, GLU>(a, s);
-    case 2: return launch_tiled<T, 32, 256, 64, 1, 4, GLU>(a, s);
+    case 0: return launch_tiled<T, 256, 256, 2, 2, GLU>(a, s);
+    case 1: return launch_tiled<T, 128, 128, 2, 2, GLU>(a, s);
+    case 2: return launch_tiled<T, 32, 256, 1, 4, GLU>(a, s);
+    case 4: return a.K % 32 == 0 ? launch_dma<T, 128, 128, 2, 2, GLU>(a, s) : MI_MOE_EUNSUPPORTED;
+    case 5: return persistent_ok(a) ? launch_persistent<T, 256, 256, 4, 2, GLU, 32, false>(a, s) : MI_MOE_EUNSUPPORTED;
+    case 6:
+      return persistent_ok(a) && a.K % 64 == 0 ? launch_persistent<T, 256, 256, 4, 2, GLU, 64, false>(a, s)
+                                               : MI_MOE_EUNSUPPORTED;
     default: return MI_MOE_EUNSUPPORTED;
   }
 }
@@ -349,9 +1093,10 @@ static bool tiled_ok(const GemmArgs& a, int in_rows_bound, bool glu) {
 }
 
 static int pick_cfg(const GemmArgs& a) {
-  long avg = a.E > 0 ? (long)a.L / a.E : a.L;
+  const long avg = a.E > 0 ? (long)a.L / a.E : a.L;  // rows per expert if the load were uniform
+  if (avg >= 192 && persistent_ok(a)) return a.K % 64 == 0 ? 6 : 5;
   if (avg >= 512) return 0;
-  if (avg >= 48) return 1;
+  if (avg >= 48) return a.K % 32 == 0 ? 4 : 1;
   return 2;
 }
 
