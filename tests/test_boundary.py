@@ -1,0 +1,235 @@
+"""CPU-side checks of the drop-in boundary: the C ABI (symbols, argument validation, error text), the
+module interface (constructor, parameter names / shapes, toggle semantics) and the eager branch, which
+must equal the oracle.  No kernel is launched here."""
+
+import ctypes
+import math
+import os
+import re
+
+import pytest
+import torch
+
+import dolomite_engine_amd as pkg
+from dolomite_engine_amd import Kernel, MoE, ParameterizedExperts, enable_kernels, is_kernel_allowed
+from dolomite_engine_amd import _lib
+from oracle import moe_oracle as oracle
+
+HEADER = _lib.HEADER_PATH
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi_moe_[a-z0-9_]+)\s*\(", text)))
+
+
+def _moe(**kw):
+    args = dict(hidden_size=32, intermediate_size=48, shared_intermediate_size=None, num_experts=8,
+                num_experts_per_tok=2, activation_function="swiglu", add_bias=False, dropout=0.0,
+                init_method="normal", initializer_range=0.02, m_width=None, num_layers=2,
+                use_padding_free_transformer=False)
+    args.update(kw)
+    return MoE(**args)
+
+
+# ---------------------------------------------------------------------------------------------------
+# C ABI
+# ---------------------------------------------------------------------------------------------------
+
+
+def test_library_is_built_and_exports_every_declared_symbol():
+    assert pkg.is_built(), "build the library first: python -c 'import __graft_entry__ as g; g.build()'"
+    declared = _declared_functions()
+    assert len(declared) >= 14
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/mi_moe.h but not exported"
+    # the Python binding table covers exactly the header
+    assert sorted(_lib.SIGNATURES) == declared
+
+
+def test_abi_version_and_error_text():
+    lib = _lib.load()
+    assert lib.mi_moe_abi_version() == _lib.ABI_VERSION
+    header = open(HEADER).read()
+    assert f"#define MI_MOE_ABI_VERSION {_lib.ABI_VERSION}" in header
+    for code, word in [(0, "ok"), (-1, "NULL"), (-2, "dimension"), (-3, "element type"), (-4, "aligned"),
+                       (-5, "workspace"), (-6, "not supported")]:
+        assert word in lib.mi_moe_strerror(code).decode()
+    assert "unknown" in lib.mi_moe_strerror(-99).decode()
+
+
+def test_argument_validation_happens_before_any_launch():
+    """Bad shapes / NULL pointers / unsupported dtypes are refused on the host (no GPU needed)."""
+    lib = _lib.load()
+    E_NULL, E_SHAPE, E_DTYPE, E_WS, E_UNSUP = -1, -2, -3, -5, -6
+    assert lib.mi_moe_router_topk_softmax(None, 4, 0, 1, _lib.BF16, None, None, None) == E_SHAPE
+    assert lib.mi_moe_router_topk_softmax(None, 4, 8, 9, _lib.BF16, None, None, None) == E_SHAPE  # k > E
+    assert lib.mi_moe_router_topk_softmax(None, 4, 8, 2, _lib.BF16, None, None, None) == E_NULL
+    assert lib.mi_moe_router_topk_softmax(None, 0, 8, 2, _lib.BF16, None, None, None) == 0  # empty input
+    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 128, 2, _lib.BF16, None, None, None, None) == E_UNSUP
+    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 8, 2, _lib.F32, None, None, None, None) == E_DTYPE
+    assert lib.mi_moe_count(None, -1, 8, None, None) == E_SHAPE
+    assert lib.mi_moe_sort_bin(None, 4, 2, 0, None, None, None, None, 0, None) == E_SHAPE
+    assert lib.mi_moe_sort_bin(None, 4, 2, 8, None, None, None, None, 0, None) == E_NULL
+    assert lib.mi_moe_sort_bin_workspace_bytes(1000, 8) == 0  # small inputs need no workspace
+    assert lib.mi_moe_sort_bin_workspace_bytes(262144, 40) == (40 * 128 + 40) * 4
+    assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 16, 0, 8, 4, 2, 0, 1, _lib.BF16, None) == E_SHAPE
+    assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 16, 8, 8, 4, 2, 0, 1, 7, None) == E_DTYPE
+    assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 16, 8, 8, 4, 2, 0, 1, _lib.BF16, None) == E_NULL
+    assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 0, 8, 8, 4, 2, 0, 1, _lib.BF16, None) == 0
+    assert lib.mi_moe_up_swiglu(None, None, None, None, None, 16, 8, 8, 4, 2, _lib.F16, None) == E_NULL
+    assert lib.mi_moe_combine(None, None, None, 4, 0, 8, _lib.BF16, None) == E_SHAPE
+    assert lib.mi_moe_combine(None, None, None, 4, 2, 8, 9, None) == E_NULL  # pointers are checked before the dtype
+    assert lib.mi_moe_up_swiglu_fp8(None, None, None, None, None, None, 16, 64, 32, 4, 2, _lib.F32, None) == E_DTYPE
+    assert lib.mi_moe_down_fp8(None, None, None, None, None, None, 16, 64, 32, 4, _lib.BF16, None) == E_NULL
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", os.path.join(os.path.dirname(_lib.LIB_PATH), "no_such_lib.so"))
+    with pytest.raises(pkg.MiMoeError, match="not found"):
+        _lib.load()
+
+
+# ---------------------------------------------------------------------------------------------------
+# toggle
+# ---------------------------------------------------------------------------------------------------
+
+
+def test_kernel_enum_matches_reference_names():
+    names = {k.name for k in Kernel}
+    assert {"scattermoe", "continuous_count_cute", "swiglu_packed_cute", "rmsnorm_cute", "flash_attention_2",
+            "mamba2_ssm", "ladder_residual_overlapped_layer"} <= names
+    assert len(names) == 16 and Kernel.scattermoe.value == "scattermoe"
+
+
+def test_enable_kernels_replaces_and_restores():
+    assert not is_kernel_allowed(Kernel.scattermoe)
+    with enable_kernels([Kernel.scattermoe]):
+        assert is_kernel_allowed(Kernel.scattermoe)
+        with enable_kernels({Kernel.rmsnorm_cute}):  # inner context replaces, it does not merge
+            assert not is_kernel_allowed(Kernel.scattermoe)
+            assert is_kernel_allowed(Kernel.rmsnorm_cute)
+        assert is_kernel_allowed(Kernel.scattermoe)
+    assert not is_kernel_allowed(Kernel.scattermoe)
+    with pytest.raises(ValueError):
+        with enable_kernels([Kernel.scattermoe]):
+            raise ValueError("boom")
+    assert not is_kernel_allowed(Kernel.scattermoe)  # restored even when the block raises
+
+
+# ---------------------------------------------------------------------------------------------------
+# module interface
+# ---------------------------------------------------------------------------------------------------
+
+
+def test_constructor_state_dict_and_init():
+    torch.manual_seed(0)
+    m = _moe(hidden_size=64, intermediate_size=96, num_experts=8, num_layers=4, initializer_range=0.02)
+    sd = m.state_dict()
+    assert {k: tuple(v.shape) for k, v in sd.items()} == {
+        "gate.weight": (8, 64), "c_fc.weight": (8, 192, 64), "c_proj.weight": (8, 64, 96)}
+    assert abs(m.c_fc.weight.std().item() - 0.02) < 2e-3
+    assert abs(m.c_proj.weight.std().item() - 0.02 / math.sqrt(2 * 4)) < 1e-3  # std / sqrt(2 * num_layers)
+    assert m.top_k == 2 and m.num_experts == 8 and isinstance(m.c_fc, ParameterizedExperts)
+    assert m.gate.weight._has_mup_learning_rate and m.c_fc.weight._has_mup_learning_rate
+    # non-GLU activation: c_fc has I rows; shared experts add two dense layers; mup scales the std
+    m2 = _moe(activation_function="gelu_pytorch_tanh", shared_intermediate_size=40, init_method="mup", m_width=4.0)
+    assert m2.c_fc.weight.shape == (8, 48, 32)
+    assert m2.c_fc_shared.weight.shape == (40, 32) and m2.c_proj_shared.weight.shape == (32, 40)
+    with pytest.raises(ValueError):
+        _moe(init_method="bogus")
+
+
+def test_num_active_parameters():
+    m = _moe(hidden_size=32, intermediate_size=48, num_experts=8, num_experts_per_tok=2)
+    total = sum(p.numel() for p in m.parameters())
+    experts = m.c_fc.weight.numel() + m.c_proj.weight.numel()
+    assert m.get_num_active_parameters() == total - experts + experts * 2 // 8
+
+
+def test_eager_branch_equals_oracle_and_handles_3d_input():
+    torch.manual_seed(1)
+    m = _moe(hidden_size=32, intermediate_size=48, num_experts=8, num_experts_per_tok=3).eval()
+    x = torch.randn(2, 9, 32)
+    pkg.clear_aux_loss()
+    with torch.no_grad():
+        y = m(x)
+    assert y.shape == x.shape and pkg.get_aux_loss() == 0 and pkg.is_aux_loss_zero(pkg.get_aux_loss())
+    ref = oracle.moe_forward(x.view(-1, 32), m.gate.weight.data, m.c_fc.weight.data, m.c_proj.weight.data, 3)
+    torch.testing.assert_close(y.view(-1, 32), ref.y, rtol=1e-5, atol=1e-6)
+
+
+def test_tiny_config_full_size_eager_equals_oracle():
+    """BASELINE config 1 (512 tokens, hidden 256, 8 experts, top-2, intermediate 512, fp32) on the CPU."""
+    w = oracle.WORKLOADS["tiny-fp32"]
+    inp = oracle.make_inputs(w)
+    m = _moe(hidden_size=w.H, intermediate_size=w.I, num_experts=w.E, num_experts_per_tok=w.k,
+             use_padding_free_transformer=True).eval()
+    with torch.no_grad():
+        m.gate.weight.copy_(inp["gate_w"]); m.c_fc.weight.copy_(inp["w_fc"]); m.c_proj.weight.copy_(inp["w_proj"])
+        y = m(inp["x"])
+    ref = oracle.moe_forward(inp["x"], inp["gate_w"], inp["w_fc"], inp["w_proj"], w.k)
+    torch.testing.assert_close(y, ref.y, rtol=1e-4, atol=1e-6)
+
+
+def test_training_mode_adds_switch_loss():
+    torch.manual_seed(2)
+    m = _moe().train()
+    pkg.clear_aux_loss()
+    x = torch.randn(1, 12, 32)
+    m(x)
+    aux = pkg.get_aux_loss()
+    assert isinstance(aux, torch.Tensor) and not pkg.is_aux_loss_zero(aux)
+    logits = m.gate(x.view(-1, 32))
+    sel = logits.topk(2, -1).indices
+    torch.testing.assert_close(aux.detach(), oracle.switch_aux_loss(logits.detach(), sel), rtol=1e-5, atol=1e-6)
+    pkg.clear_aux_loss()
+
+
+def test_router_logit_bias_is_added_before_topk():
+    torch.manual_seed(3)
+    m = _moe().eval()
+    m.router_logit_bias = torch.tensor([9.0, 0, 0, 0, 0, 0, 0, 9.0])
+    x = torch.randn(20, 32).view(1, 20, 32)
+    with torch.no_grad():
+        _, _, sel = m._compute_routing_weights(x.view(-1, 32))
+    assert set(sel.flatten().tolist()) == {0, 7}
+    assert "router_logit_bias" not in m.state_dict()  # not part of the checkpoint format
+
+
+def test_kernel_branch_has_no_cpu_fallback():
+    m = _moe().eval()
+    x = torch.randn(1, 4, 32)
+    with torch.no_grad(), enable_kernels([Kernel.scattermoe]):
+        with pytest.raises(ValueError, match="GPU"):
+            m(x)
+
+
+def test_fp8_quantisation_eager_path():
+    torch.manual_seed(4)
+    m = _moe(hidden_size=64, intermediate_size=32).eval()
+    x = torch.randn(1, 10, 64)
+    w_fc, w_proj = m.c_fc.weight.data.clone(), m.c_proj.weight.data.clone()
+    m.quantize_expert_weights_fp8()
+    assert m.c_fc.weight is None and m.c_fc.weight_q.dtype == torch.float8_e4m3fn
+    assert m.c_fc.weight_scale.shape == (8, 64) and m.c_proj.weight_scale.shape == (8, 64)
+    q_fc, s_fc = oracle.quantize_fp8_per_channel(w_fc)
+    q_pj, s_pj = oracle.quantize_fp8_per_channel(w_proj)
+    assert torch.equal(m.c_fc.weight_q.view(torch.uint8), q_fc.view(torch.uint8))
+    with torch.no_grad():
+        y = m(x)
+    ref = oracle.moe_forward(x.view(-1, 64), m.gate.weight.data, q_fc, q_pj, 2, w_fc_scale=s_fc, w_proj_scale=s_pj)
+    torch.testing.assert_close(y.view(-1, 64), ref.y, rtol=1e-4, atol=1e-6)
+
+
+def test_activation_registry():
+    assert pkg.is_glu("swiglu") and pkg.is_glu("geglu") and not pkg.is_glu("gelu")
+    act = pkg.get_activation_function("swiglu")
+    h = torch.randn(5, 8)
+    torch.testing.assert_close(act(h), h[:, :4] * torch.nn.functional.silu(h[:, 4:]))
+    assert isinstance(pkg.get_activation_function(None), torch.nn.Identity)
+    with pytest.raises(ValueError):
+        pkg.get_activation_function("no_such_act")
