@@ -19,6 +19,7 @@
 //   * the per-channel scale, SwiGLU and the 8-byte packed store happen in the epilogue.
 #include "common.h"
 
+
 template <typename T> struct Mfma16;
 template <> struct Mfma16<bf16_t> {
   typedef bf16x8 vec;
@@ -164,6 +165,214 @@ __global__ __launch_bounds__(256) void decode_fp8_kernel(DecodeArgs a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Streaming variant: weights and activations reach the matrix cores through per-wave LDS rings filled
+// by DMA (global_load_lds_dwordx4).
+//
+// In the kernel above the lane -> address map is dictated by the MFMA operand layout (lane = 16*q + r
+// reads row r): neighbouring lanes touch different rows, every 16-byte access is its own cache-line
+// lookup, and the address path, not HBM, sets the pace.  Here the global side is laid out for the
+// memory system -- 8 neighbouring lanes read one full 128-byte line of a weight row, 16 neighbouring
+// lanes 256 bytes of an activation row -- and the MFMA layout is recovered by where the ds_reads look.
+//
+//   wave       = 32 weight rows over the whole K (SwiGLU: 16 up + 16 gate rows -> 16 output channels);
+//                the four waves of a workgroup are independent: no barrier, no cross-wave sum, and two
+//                workgroups fit on a CU
+//   ring       = NS stages per wave; stage = [32 rows][128 B] fp8 weights + [XT rows][256 B] activations
+//   stage      : lane (r, q) takes k [32q, 32q+32) of the stage: per 16-row block two 16-byte weight
+//                reads and four MFMA 16x16x32, plus four 16-byte activation reads
+//   activations: an expert with at most 8 rows (the decode case) runs one pass with XT = 8 and a
+//                three-stage ring (MFMA columns 8..15 mirror 0..7 and are never stored); more rows run
+//                passes of 16 with a two-stage ring.  Only ceil(rows/4)*4 rows are fetched.
+// Measured against an empty kernel that merely streams the same rows (no LDS reads, no MFMA) this kernel
+// is within ~10 %: at this size (0.4 - 0.7 GB per launch) launch ramp and tail, not the inner loop,
+// separate it from the 7.3 TB/s a long-running stream reaches on this part.
+// Needs K % 128 == 0; other shapes take the kernel above.
+// ------------------------------------------------------------------------------------------------
+
+// LDS per wave: three stages of [32 x 128] weights + [8 x 256] activations (= two stages with 16 rows)
+#define DEC_WAVE_LDS (3 * (32 * 128 + 8 * 256))
+
+__device__ __forceinline__ constexpr int dec_waitcnt(int vm, int lgkm) {
+  return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8);
+}
+
+template <int V> struct dec_int { static constexpr int value = V; };
+
+template <typename T, bool GLU>
+__global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
+  constexpr int KCH = 128;                       // k per ring stage
+  constexpr int WR = GLU ? 2 : 1;
+  constexpr int CHW = GLU ? 16 : 32;             // output channels per wave
+  constexpr int NWI = 4;                         // weight DMA instructions per stage (8 rows x 128 B each)
+  constexpr int W_BYTES = 32 * KCH;
+  constexpr int NM = KCH / 32;                   // MFMA k-steps per stage
+  typedef typename Mfma16<T>::vec frag_t;
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  typedef const __attribute__((address_space(1))) void* glb_ptr_t;
+  extern __shared__ __attribute__((aligned(16))) unsigned char dsm[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, q = lane >> 4;
+  const int expert = blockIdx.x / a.groups_per_expert;
+  const int grp = blockIdx.x - expert * a.groups_per_expert;
+  const int row_begin = expert ? a.expert_offsets[expert - 1] : 0;
+  const int row_end = a.expert_offsets[expert];
+  if (row_begin >= row_end) return;  // nothing routed here: the expert's weights stay untouched
+  const int n0 = (grp * 4 + wave) * CHW;
+  if (n0 >= a.N) return;             // whole wave past the last channel (waves do not synchronise)
+
+  unsigned char* ring = dsm + wave * DEC_WAVE_LDS;
+
+  // weight DMA: instruction j fills ring rows [8j, 8j+8): lane -> row 8j + lane/8, slot lane%8 holding
+  // logical chunk slot ^ ((row >> 1) & 7)  (conflict-free ds_read_b128 on the 64-bank LDS)
+  const unsigned char* wexp = a.wq + (size_t)expert * WR * a.N * a.K;
+  uint32_t woff[NWI];
+#pragma unroll
+  for (int j = 0; j < NWI; ++j) {
+    const int t = 8 * j + (lane >> 3);                      // ring row 0..31
+    int ch;                                                 // weight row inside the expert
+    if (GLU) {
+      ch = t < 16 ? n0 + t : a.N + n0 + (t - 16);
+      const int lim = (t < 16 ? a.N : 2 * a.N) - 1;
+      if (ch > lim) ch = lim;                               // channel tail re-reads the last row; never stored
+    } else {
+      ch = n0 + t;
+      if (ch > a.N - 1) ch = a.N - 1;
+    }
+    woff[j] = (uint32_t)ch * (uint32_t)a.K + ((lane & 7) ^ ((t >> 1) & 7)) * 16;
+  }
+
+  const int nst = a.K / KCH;
+  const T* __restrict__ xin = static_cast<const T*>(a.in);
+  T* __restrict__ out = static_cast<T*>(a.out);
+
+  // One pass over K for the activation rows [g0, g0 + XT): ring of NS stages, NX activation DMA
+  // instructions per stage (4 rows each).
+  auto pass = [&](int g0, auto xt_tag, auto ns_tag, auto nx_tag) {
+    constexpr int XT = decltype(xt_tag)::value;
+    constexpr int NS = decltype(ns_tag)::value;
+    constexpr int NX = decltype(nx_tag)::value;
+    constexpr int STAGE = W_BYTES + XT * KCH * 2;
+    constexpr int NDMA = NWI + NX;
+    static_assert(NS * STAGE <= DEC_WAVE_LDS, "ring does not fit");
+    // activation DMA: instruction j fills ring rows [4j, 4j+4): lane -> row 4j + lane/16, slot lane%16
+    // holding logical chunk slot ^ row
+    const T* xsrc[NX];
+#pragma unroll
+    for (int j = 0; j < NX; ++j) {
+      const int t = 4 * j + (lane >> 4);
+      int srow = g0 + t;
+      if (srow > row_end - 1) srow = row_end - 1;           // short pass re-reads the last row; never stored
+      const int src = a.gather ? a.sorted_scattered[srow] / a.kdiv : srow;
+      xsrc[j] = xin + (size_t)src * a.K + (((lane & 15) ^ t) * 8);
+    }
+    auto dma_stage = [&](int st, int slot) {
+      const int stc = st < nst ? st : nst - 1;               // surplus rounds re-fetch the last stage
+      unsigned char* dst = ring + slot * STAGE;
+      const unsigned char* wk = wexp + (size_t)stc * KCH;
+#pragma unroll
+      for (int j = 0; j < NWI; ++j)
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(wk + woff[j]), (lds_ptr_t)(dst + j * 1024), 16, 0, 0);
+#pragma unroll
+      for (int j = 0; j < NX; ++j)
+        __builtin_amdgcn_global_load_lds((glb_ptr_t)(xsrc[j] + (size_t)stc * KCH),
+                                         (lds_ptr_t)(dst + W_BYTES + j * 1024), 16, 0, 0);
+    };
+
+    f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    const int xr = r & (XT - 1);                             // XT = 8: columns 8..15 mirror 0..7
+#pragma unroll
+    for (int p = 0; p < NS; ++p) dma_stage(p, p);
+    int slot = 0;
+    for (int i = 0; i < nst; ++i) {
+      __builtin_amdgcn_s_waitcnt(dec_waitcnt((NS - 1) * NDMA, 15));  // stage i has landed
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      const unsigned char* ws = ring + slot * STAGE;
+      const unsigned char* xs = ws + W_BYTES;
+      frag_t xb[NM];
+#pragma unroll
+      for (int m = 0; m < NM; ++m)
+        xb[m] = __builtin_bit_cast(frag_t,
+                                   *reinterpret_cast<const u32x4*>(xs + xr * (KCH * 2) + (((q * NM + m) ^ xr) * 16)));
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int t = 16 * b + r;
+#pragma unroll
+        for (int h = 0; h < NM / 2; ++h) {
+          const u32x4 wv =
+              *reinterpret_cast<const u32x4*>(ws + t * KCH + (((q * (NM / 2) + h) ^ ((t >> 1) & 7)) * 16));
+          acc[b] = Mfma16<T>::run(Mfma16<T>::widen(wv[0], wv[1]), xb[2 * h], acc[b]);
+          acc[b] = Mfma16<T>::run(Mfma16<T>::widen(wv[2], wv[3]), xb[2 * h + 1], acc[b]);
+        }
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(dec_waitcnt(63, 0));                // my reads of this slot are done
+      dma_stage(i + NS, slot);
+      slot = slot + 1 == NS ? 0 : slot + 1;
+    }
+    __builtin_amdgcn_s_waitcnt(dec_waitcnt(0, 0));
+
+    // acc[b][i]: weight row 16b + 4q + i of this wave, activation row g0 + r
+    if (r < XT && g0 + r < row_end) {
+      const int orow = a.scatter ? a.sorted_scattered[g0 + r] : g0 + r;
+      if (GLU) {
+        const int col = n0 + 4 * q;
+        if (col < a.N) {
+          const float* sp = a.scale + (size_t)expert * WR * a.N + col;
+          const f32x4 scu = *reinterpret_cast<const f32x4*>(sp);
+          const f32x4 scg = *reinterpret_cast<const f32x4*>(sp + a.N);
+          float v[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = (acc[0][i] * scu[i]) * silu_f32(acc[1][i] * scg[i]);
+          const u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+          *reinterpret_cast<u32x2*>(out + (size_t)orow * a.N + col) = p;
+        }
+      } else {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const int col = n0 + 16 * b + 4 * q;
+          if (col < a.N) {
+            const f32x4 sc = *reinterpret_cast<const f32x4*>(a.scale + (size_t)expert * a.N + col);
+            const u32x2 p = {pack2<T>(acc[b][0] * sc[0], acc[b][1] * sc[1]),
+                             pack2<T>(acc[b][2] * sc[2], acc[b][3] * sc[3])};
+            *reinterpret_cast<u32x2*>(out + (size_t)orow * a.N + col) = p;
+          }
+        }
+      }
+    }
+  };
+
+  const int n_rows = row_end - row_begin;
+  if (n_rows <= 4) {
+    pass(row_begin, dec_int<8>{}, dec_int<3>{}, dec_int<1>{});
+  } else if (n_rows <= 8) {
+    pass(row_begin, dec_int<8>{}, dec_int<3>{}, dec_int<2>{});
+  } else {
+    for (int g0 = row_begin; g0 < row_end; g0 += 16) pass(g0, dec_int<16>{}, dec_int<2>{}, dec_int<4>{});
+  }
+}
+
+template <typename T, bool GLU>
+static int launch_decode_stream(DecodeArgs a, hipStream_t s) {
+  constexpr int CH = 4 * (GLU ? 16 : 32);
+  constexpr int LDS = 4 * DEC_WAVE_LDS;
+  auto kern = decode_fp8_stream_kernel<T, GLU>;
+  if (LDS > 64 * 1024) {
+    hipError_t e =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+    if (e != hipSuccess) return (int)e;
+  }
+  a.groups_per_expert = mi_ceil_div(a.N, CH);
+  long grid = (long)a.E * a.groups_per_expert;
+  if (grid > 0x7fffffffL) return MI_MOE_ESHAPE;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), LDS, s, a);
+  return mi_launch_status();
+}
+
 template <typename T, bool GLU, int KSPLIT>
 static int launch_decode(DecodeArgs a, hipStream_t s) {
   constexpr int NTB = 4 / KSPLIT;
@@ -176,6 +385,8 @@ static int launch_decode(DecodeArgs a, hipStream_t s) {
 
 template <typename T, bool GLU>
 static int dispatch_decode(const DecodeArgs& a, hipStream_t s) {
+  // the streaming kernel needs whole 128-wide K stages and 32-bit weight offsets inside one expert
+  if (a.K % 128 == 0 && a.K >= 512 && (double)(GLU ? 2 : 1) * a.N * a.K < 4.0e9) return launch_decode_stream<T, GLU>(a, s);
   if (a.K >= 2048) return launch_decode<T, GLU, 4>(a, s);
   if (a.K >= 1024) return launch_decode<T, GLU, 2>(a, s);
   return launch_decode<T, GLU, 1>(a, s);
