@@ -35,6 +35,80 @@ __device__ __forceinline__ uint32_t router_ordered_key(float v) {
 
 #define ROUTER_KMAX 8
 
+// Epilogue for one group of 16 tokens: lane (r = token, q) holds acc[eb][i] = logit of expert
+// 16*eb + 4*q + i.  Rounds to the model dtype, adds the optional bias, optionally stores the logits,
+// selects the top-k (value descending, expert ascending) and writes the softmax of the k winners.
+template <typename T>
+__device__ __forceinline__ void router_epilogue(const f32x4 (&acc)[4], int t, bool tvalid, int q,
+                                                const float* __restrict__ bias, int E, int k,
+                                                T* __restrict__ logits_out, T* __restrict__ gates,
+                                                int32_t* __restrict__ idx) {
+  uint64_t keys[16];
+  float vals[16];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int e = eb * 16 + 4 * q + i;
+      float v = Elt<T>::round(acc[eb][i]);
+      if (bias != nullptr && e < E) v = Elt<T>::round(v + bias[e]);
+      vals[eb * 4 + i] = v;
+      keys[eb * 4 + i] = e < E ? (((uint64_t)router_ordered_key(v) << 32) | (uint32_t)(~(uint32_t)e)) : 0ull;
+      if (logits_out != nullptr && tvalid && e < E) Elt<T>::store(logits_out + (size_t)t * E + e, v);
+    }
+  }
+  float wv[ROUTER_KMAX];
+  int wi[ROUTER_KMAX];
+#pragma unroll
+  for (int j = 0; j < ROUTER_KMAX; ++j) {
+    wv[j] = 0.f;
+    wi[j] = 0;
+    if (j < k) {
+      uint64_t best = 0ull;
+      float bv = 0.f;
+#pragma unroll
+      for (int c = 0; c < 16; ++c) {
+        if (keys[c] > best) {
+          best = keys[c];
+          bv = vals[c];
+        }
+      }
+#pragma unroll
+      for (int off = 16; off <= 32; off <<= 1) {
+        uint32_t lo = __shfl_xor((uint32_t)best, off, MI_WAVE);
+        uint32_t hi = __shfl_xor((uint32_t)(best >> 32), off, MI_WAVE);
+        float ov = __shfl_xor(bv, off, MI_WAVE);
+        uint64_t o = ((uint64_t)hi << 32) | lo;
+        if (o > best) {
+          best = o;
+          bv = ov;
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 16; ++c)
+        if (keys[c] == best) keys[c] = 0ull;
+      wv[j] = bv;
+      wi[j] = (int)(~(uint32_t)best);
+    }
+  }
+  if (q == 0 && tvalid) {
+    float p[ROUTER_KMAX];
+    float denom = 0.f;
+#pragma unroll
+    for (int j = 0; j < ROUTER_KMAX; ++j) {
+      p[j] = j < k ? expf(wv[j] - wv[0]) : 0.f;
+      denom += p[j];
+    }
+#pragma unroll
+    for (int j = 0; j < ROUTER_KMAX; ++j) {
+      if (j < k) {
+        Elt<T>::store(gates + (size_t)t * k + j, p[j] / denom);
+        idx[(size_t)t * k + j] = wi[j];
+      }
+    }
+  }
+}
+
 template <typename T, int TG>
 __global__ __launch_bounds__(256) void router_fused_kernel(const T* __restrict__ x, const T* __restrict__ gw,
                                                            const float* __restrict__ bias, int Trows, int H, int E,
@@ -102,77 +176,82 @@ __global__ __launch_bounds__(256) void router_fused_kernel(const T* __restrict__
 #pragma unroll
   for (int g = 0; g < TG; ++g) {
     const int t = tok0 + g * 16 + r;
-    const bool tvalid = t < Trows;
-    uint64_t keys[16];
-    float vals[16];
+    f32x4 a4[4];
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) a4[eb] = acc[eb][g];
+    router_epilogue<T>(a4, t, t < Trows, q, bias, E, k, logits_out, gates, idx);
+  }
+}
+
+// Few tokens (decode): one workgroup of 16 waves per group of 16 tokens; the waves split K (wave w takes
+// the 64-wide K steps w, w+16, ...) and their partial logits meet in LDS, so that the latency of walking
+// H is paid once per 16th of the row instead of once per row.
+template <typename T>
+__global__ __launch_bounds__(1024) void router_fused_small_kernel(const T* __restrict__ x, const T* __restrict__ gw,
+                                                                  const float* __restrict__ bias, int Trows, int H,
+                                                                  int E, int k, T* __restrict__ logits_out,
+                                                                  T* __restrict__ gates, int32_t* __restrict__ idx) {
+  typedef typename RMfma<T>::vec frag_t;
+  __shared__ f32x4 red[16][4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int tok0 = blockIdx.x * 16;
+  int t = tok0 + r;
+  const bool tvalid = t < Trows;
+  const T* xrow = x + (size_t)(tvalid ? t : Trows - 1) * H;
+  const T* wrow[4];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) {
+    int e = eb * 16 + r;
+    if (e > E - 1) e = E - 1;
+    wrow[eb] = gw + (size_t)e * H;
+  }
+  f32x4 acc[4];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) acc[eb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int k0 = wave * 64; k0 < H; k0 += 16 * 64) {
+    const int kpos = k0 + q * 16;
+    const bool valid = kpos < H;  // the MFMA runs on all lanes: out-of-range k contributes zeros
+    u32x4 x0 = {0u, 0u, 0u, 0u}, x1 = {0u, 0u, 0u, 0u};
+    if (valid) {
+      x0 = *reinterpret_cast<const u32x4*>(xrow + kpos);
+      x1 = *reinterpret_cast<const u32x4*>(xrow + kpos + 8);
+    }
 #pragma unroll
     for (int eb = 0; eb < 4; ++eb) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int e = eb * 16 + 4 * q + i;
-        float v = Elt<T>::round(acc[eb][g][i]);
-        if (bias != nullptr && e < E) v = Elt<T>::round(v + bias[e]);
-        vals[eb * 4 + i] = v;
-        keys[eb * 4 + i] = e < E ? (((uint64_t)router_ordered_key(v) << 32) | (uint32_t)(~(uint32_t)e)) : 0ull;
-        if (logits_out != nullptr && tvalid && e < E) Elt<T>::store(logits_out + (size_t)t * E + e, v);
+      u32x4 w0 = {0u, 0u, 0u, 0u}, w1 = {0u, 0u, 0u, 0u};
+      if (valid) {
+        w0 = *reinterpret_cast<const u32x4*>(wrow[eb] + kpos);
+        w1 = *reinterpret_cast<const u32x4*>(wrow[eb] + kpos + 8);
       }
+      acc[eb] = RMfma<T>::run(__builtin_bit_cast(frag_t, w0), __builtin_bit_cast(frag_t, x0), acc[eb]);
+      acc[eb] = RMfma<T>::run(__builtin_bit_cast(frag_t, w1), __builtin_bit_cast(frag_t, x1), acc[eb]);
     }
-    float wv[ROUTER_KMAX];
-    int wi[ROUTER_KMAX];
+  }
 #pragma unroll
-    for (int j = 0; j < ROUTER_KMAX; ++j) {
-      wv[j] = 0.f;
-      wi[j] = 0;
-      if (j < k) {
-        uint64_t best = 0ull;
-        float bv = 0.f;
+  for (int eb = 0; eb < 4; ++eb) red[wave][eb][lane] = acc[eb];
+  __syncthreads();
+  if (wave == 0) {
+    // fixed summation order (wave 0, 1, ..., 15): the logits do not depend on scheduling
 #pragma unroll
-        for (int c = 0; c < 16; ++c) {
-          if (keys[c] > best) {
-            best = keys[c];
-            bv = vals[c];
-          }
-        }
-#pragma unroll
-        for (int off = 16; off <= 32; off <<= 1) {
-          uint32_t lo = __shfl_xor((uint32_t)best, off, MI_WAVE);
-          uint32_t hi = __shfl_xor((uint32_t)(best >> 32), off, MI_WAVE);
-          float ov = __shfl_xor(bv, off, MI_WAVE);
-          uint64_t o = ((uint64_t)hi << 32) | lo;
-          if (o > best) {
-            best = o;
-            bv = ov;
-          }
-        }
-#pragma unroll
-        for (int c = 0; c < 16; ++c)
-          if (keys[c] == best) keys[c] = 0ull;
-        wv[j] = bv;
-        wi[j] = (int)(~(uint32_t)best);
-      }
+    for (int eb = 0; eb < 4; ++eb) {
+      f32x4 sum = red[0][eb][lane];
+      for (int w = 1; w < 16; ++w) sum += red[w][eb][lane];
+      acc[eb] = sum;
     }
-    if (q == 0 && tvalid) {
-      float p[ROUTER_KMAX];
-      float denom = 0.f;
-#pragma unroll
-      for (int j = 0; j < ROUTER_KMAX; ++j) {
-        p[j] = j < k ? expf(wv[j] - wv[0]) : 0.f;
-        denom += p[j];
-      }
-#pragma unroll
-      for (int j = 0; j < ROUTER_KMAX; ++j) {
-        if (j < k) {
-          Elt<T>::store(gates + (size_t)t * k + j, p[j] / denom);
-          idx[(size_t)t * k + j] = wi[j];
-        }
-      }
-    }
+    router_epilogue<T>(acc, t, tvalid, q, bias, E, k, logits_out, gates, idx);
   }
 }
 
 template <typename T>
 static int launch_router(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
                          void* logits_out, void* gates, int32_t* idx, hipStream_t s) {
+  if (T_ <= 1024) {  // fewer than 4 workgroups' worth of tokens for the streaming kernel: split K instead
+    hipLaunchKernelGGL((router_fused_small_kernel<T>), dim3(mi_ceil_div(T_, 16)), dim3(1024), 0, s,
+                       static_cast<const T*>(x), static_cast<const T*>(gw), bias, T_, H, E, k,
+                       static_cast<T*>(logits_out), static_cast<T*>(gates), idx);
+    return mi_launch_status();
+  }
   constexpr int TG = 2;
   dim3 grid(mi_ceil_div(T_, 4 * 16 * TG)), block(256);
   hipLaunchKernelGGL((router_fused_kernel<T, TG>), grid, block, 0, s, static_cast<const T*>(x),

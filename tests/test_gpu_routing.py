@@ -103,7 +103,8 @@ def test_count(device, L, E):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,H,E,k,bias", [(1, 64, 8, 2, False), (15, 32, 8, 8, False), (200, 256, 40, 8, True),
                                           (1000, 1024, 32, 8, False), (64, 4096, 64, 6, False),
-                                          (333, 1536, 40, 8, True), (130, 48, 5, 1, False)])
+                                          (333, 1536, 40, 8, True), (130, 48, 5, 1, False),
+                                          (2500, 256, 40, 8, True), (4099, 512, 64, 6, False)])
 def test_router_fused(device, dtype, T, H, E, k, bias):
     ops = _ops()
     g = torch.Generator().manual_seed(T + H + E)
