@@ -29,6 +29,15 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
+# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
+# of this script (scaled by what the counters read for the 256 MiB copy of --pmc-calibration: x2.000
+# for FETCH_SIZE, x1.000 for WRITE_SIZE); the summaries are under profiles/.  A counter cannot be read
+# from inside this process, so the figures are recorded here and are null for other workloads.
+MEASURED_TRAFFIC_BYTES = {
+    "granite-3b-a800m": 1464.2e6 + 268.6e6,   # up-projection GEMM: fetch + write
+    "decode-fp8": 758.0e6 + 1.1e6,            # fp8 up-projection: fetch + write
+}
+
 
 class StageTimer:
     """HIP events (torch.cuda.Event on the current stream, which is the stream the kernels are
@@ -128,6 +137,9 @@ def main():
     ap.add_argument("--workload", default="granite-3b-a800m")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=None)
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run one 256 MiB device-to-device copy so that a rocprofv3 --pmc FETCH_SIZE / "
+                         "WRITE_SIZE run of this command contains a kernel of known traffic to scale by")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -152,6 +164,13 @@ def main():
     x = inputs["x"].to(device)
     T, H, E, k, I = w.T, w.H, w.E, w.k, w.I
     L = T * k
+
+    if args.pmc_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=device).random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     with torch.no_grad(), enable_kernels([Kernel.scattermoe]):
         for _ in range(args.warmup):
@@ -184,14 +203,15 @@ def main():
         up_bytes = touched * (2 * I * H) + touched * 2 * I * 4 + T * H * 2 + L * I * 2 + L * 4 + E * 4
         ach = up_bytes / (stages[up_name] * 1e-3) / 1e9
         roofline = {"kernel": up_name, "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": ach / PEAK_HBM_GBS, "traffic": None, "algorithmic_bytes": up_bytes,
+                    "frac": ach / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+                    "algorithmic_bytes": up_bytes,
                     "avg_launch_ms": stages[up_name]}
     else:
         up_name = "up_swiglu"
         up_flops = 4.0 * L * H * I
         ach = up_flops / (stages[up_name] * 1e-3) / 1e12
         roofline = {"kernel": up_name, "bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS,
-                    "unit": "TFLOP/s", "frac": ach / PEAK_BF16_TFLOPS, "traffic": None,
+                    "unit": "TFLOP/s", "frac": ach / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
                     "algorithmic_flops": up_flops, "avg_launch_ms": stages[up_name]}
         if "scattered_gemm" in stages:
             down = 2.0 * L * H * I / (stages["scattered_gemm"] * 1e-3) / 1e12
