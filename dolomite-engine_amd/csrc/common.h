@@ -22,11 +22,12 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 
+// fp32 -> bf16, round to nearest even, NaN stays NaN: one v_cvt_pk_bf16_f32 (two elements per instruction)
+typedef __bf16 mi_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float mi_f32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  const __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(uint16_t, b);
 }
 
 template <typename T> struct Elt;
@@ -53,7 +54,8 @@ template <> struct Elt<f16_t> {
 // pack two floats into two 16-bit elements of type T (low half = a)
 template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
 template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
-  return (uint32_t)float_to_bf16_bits(a) | ((uint32_t)float_to_bf16_bits(b) << 16);
+  const mi_f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, mi_bf16x2));
 }
 template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
   f16_t ha = (f16_t)a, hb = (f16_t)b;

@@ -411,6 +411,26 @@ __device__ __forceinline__ constexpr int waitcnt_imm(int vm, int lgkm) {
   return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8);
 }
 
+// One DMA instruction: every lane moves 16 bytes from (scalar base + its 32-bit byte offset) to LDS; the
+// 64 destinations are the contiguous run starting at the LDS byte address in M0.  Written as inline
+// assembly on purpose: for the builtin the compiler assumes that any later LDS read may alias the DMA write
+// and puts "s_waitcnt vmcnt(0)" in front of it, which drains the prefetch ring every K slice.  Here the
+// ordering is done by hand (s_waitcnt immediates before the barrier that publishes a stage).
+// The offset register is read when the instruction issues, but the compiler treats a register named by an
+// assembly statement as busy until vmcnt reaches 0 and waits before overwriting it: callers pass offsets
+// that live in registers of their own for a whole tile, never a per-slice temporary.  TAG keeps otherwise
+// identical statements in the two arms of a branch from being merged back into one with a selected
+// (temporary) operand.
+template <int TAG>
+__device__ __forceinline__ void dma16_to_lds(const void* base, uint32_t byte_off, uint32_t lds_addr) {
+  if (TAG == 0)
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(byte_off), "s"(base)
+                 : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 ; next tile" : : "s"(lds_addr), "v"(byte_off), "s"(base)
+                 : "memory", "m0");
+}
+
 template <typename T, int BM, int BNW, int WM, int WN, bool GLU>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GemmArgs a) {
   constexpr int BK = 32;
@@ -615,11 +635,19 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GemmArgs 
 // Tile order: workgroup b serves XCD b % 8 (hardware deals workgroup ids round-robin to the XCDs); the
 // XCD's contiguous tile range is dealt to its workgroups in turn, so at any moment the CUs of one XCD
 // work on neighbouring tiles (same expert weights, shared activation rows) out of one L2.
+//
+// PP selects how the eight waves share a SIMD's matrix pipe.  Without it all waves run the same phase
+// and meet at one barrier per K slice: the two waves of a SIMD then stall together (barrier, LDS
+// latency, DMA issue) and the pipe idles.  With it the waves form two groups that alternate between a
+// memory phase and a matrix phase (see pp_slice); measured on the 32768-token Granite-3B shape that
+// takes the K loop from about 65 % to about 93 % matrix-pipe occupancy in cycles.  (With random operands
+// the chip then lowers its clock to stay inside its power limit, so wall time improves less than the
+// cycle count.)
 // ------------------------------------------------------------------------------------------------
 
 #define PERSIST_MAX_E 256
 
-template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool SCHED>
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool PP>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(GemmArgs a) {
   static_assert(BK == 32 || BK == 64, "BK");
   constexpr int NSTAGE = BK == 32 ? 4 : 2;   // ring of 128 KiB either way
@@ -641,9 +669,6 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   constexpr int MB = WTM / 32, NB = WTN / 32;
   constexpr int OB = GLU ? NB / 2 : NB;      // output column blocks per wave
   constexpr int NMFMA = MB * NB;
-  constexpr int NRD = MB + NB;
-  constexpr int RD_PER = (NRD + NMFMA - 1) / NMFMA;
-  constexpr int LD_PER = (NLD + NMFMA - 1) / NMFMA;
   static_assert(BM % (16 * NW) == 0 && BNW % (16 * NW) == 0 && NW % 2 == 0, "tile/wave shape");
   static_assert(OB % EPI_OB == 0, "epilogue pass shape");
   static_assert((NSTAGE - 1) * NLD <= 63, "vmcnt range");
@@ -764,13 +789,15 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     const size_t kbytes = (size_t)kt * BK * sizeof(T);
     const unsigned char* xs = xbase + kbytes;
     const unsigned char* ws = (from_next ? next.wbase : cur.wbase) + kbytes;
+    const uint32_t stage_lds = (uint32_t)(size_t)(lds_ptr_t)smem_raw + stage * STAGE_BYTES;
+    // activation rows fill stage rows [0, BM), weight rows [BM, BM + BNW)
+    auto grp = [&](int j) { return j < NXLD ? (j * NW + wave) : (BM / RPI + (j - NXLD) * NW + wave); };
+    if (from_next) {
 #pragma unroll
-    for (int j = 0; j < NLD; ++j) {
-      // activation rows fill stage rows [0, BM), weight rows [BM, BM + BNW)
-      const int grp = j < NXLD ? (j * NW + wave) : (BM / RPI + (j - NXLD) * NW + wave);
-      unsigned char* dst = smem_raw + stage * STAGE_BYTES + grp * 1024;
-      const uint32_t o = from_next ? next.off[j] : cur.off[j];
-      __builtin_amdgcn_global_load_lds((glb_ptr_t)((j < NXLD ? xs : ws) + o), (lds_ptr_t)dst, 16, 0, 0);
+      for (int j = 0; j < NLD; ++j) dma16_to_lds<1>(j < NXLD ? xs : ws, next.off[j], stage_lds + grp(j) * 1024);
+    } else {
+#pragma unroll
+      for (int j = 0; j < NLD; ++j) dma16_to_lds<0>(j < NXLD ? xs : ws, cur.off[j], stage_lds + grp(j) * 1024);
     }
   };
 
@@ -830,13 +857,6 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     for (int st = 0; st < STEPS - 1; ++st) {
       read_frags(cur, st + 1, (st + 1) & 1);
       mfma_step(st & 1);
-      if (SCHED) {
-#pragma unroll
-        for (int i = 0; i < NMFMA; ++i) {
-          __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(SG_DS_RD, RD_PER, 0);
-        }
-      }
       __builtin_amdgcn_sched_barrier(0);
     }
     asm volatile("" ::: "memory");
@@ -847,14 +867,31 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     read_frags(nxt, 0, 0);
     dma_slice(tcur, tnext, from_next, kload, cur);
     mfma_step((STEPS - 1) & 1);
-    if (SCHED) {
-#pragma unroll
-      for (int i = 0; i < NMFMA; ++i) {
-        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(SG_DS_RD, RD_PER, 0);
-        __builtin_amdgcn_sched_group_barrier(SG_VMEM_RD, LD_PER, 0);
-      }
-    }
+    __builtin_amdgcn_sched_barrier(0);
+    ++g;
+  };
+  // Ping-pong form of one K slice (PP; BK = 32, four stages).  The waves with wn == 0 and those with
+  // wn == 1 -- one of each per SIMD -- run this same code one phase apart (see the tile loop): while one group
+  // issues its 2 * NMFMA matrix instructions back to back out of registers, the other reads its fragments of the
+  // slice from LDS and issues its share of the DMA for slice g + 3 into the stage both groups have finished
+  // reading.  Every phase ends in a workgroup barrier; at each barrier one group has just issued its last MFMA
+  // and the other has its operands in registers, so the matrix pipe of the SIMD never waits for LDS, DMA or the
+  // barrier itself.
+  auto pp_slice = [&](const TileSrc& tcur, const TileSrc& tnext, bool from_next, int kload) {
+    const int cur = g & (NSTAGE - 1), fill = (g + NSTAGE - 1) & (NSTAGE - 1);
+    read_frags(cur, 0, 0);
+    read_frags(cur, 1, 1);
+    dma_slice(tcur, tnext, from_next, kload, fill);
+    asm volatile("" ::: "memory");
+    // own DMA of slice g + 1 has landed (slices g + 2 and g + 3 stay in flight); fragments are in registers
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm((NSTAGE - 2) * NLD, 0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_step(0);
+    mfma_step(1);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     ++g;
   };
@@ -866,6 +903,17 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     // scratch row r keeps its EPI_CPR 16-byte chunks at slots chunk ^ swz(r): the 8-byte writes of a
     // wave (32 rows, one chunk) and the 16-byte read-back both spread over all banks
     auto swz = [](int r) { return EPI_CPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3); };
+    constexpr int RPP = 64 / EPI_CPR;  // rows per read-back pass
+    // destination rows of everything this lane will store, fetched up front: one memory latency per tile
+    // instead of one per store
+    int orow_of[MB][32 / RPP];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int it = 0; it < 32 / RPP; ++it) {
+        const int row = tc.row_begin + wm * WTM + mb * 32 + it * RPP + lane / EPI_CPR;
+        orow_of[mb][it] = (a.scatter && row < tc.row_end) ? a.sorted_scattered[row] : row;
+      }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
@@ -893,7 +941,6 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
           }
         }
         // read back: lane -> row it*RPP + lane/EPI_CPR, 16-byte chunk lane%EPI_CPR
-        constexpr int RPP = 64 / EPI_CPR;  // rows per read-back pass
         const int cchunk = lane % EPI_CPR;
         const int col = tc.nt * BN + (GLU ? wn * (WTN / 2) : wn * WTN) + og * EPI_COLS + cchunk * 8;
 #pragma unroll
@@ -901,10 +948,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
           const int r = it * RPP + lane / EPI_CPR;
           const u32x4 val = *reinterpret_cast<const u32x4*>(scratch + r * (EPI_COLS * 2) + ((cchunk ^ swz(r)) * 16));
           const int row = tc.row_begin + wm * WTM + mb * 32 + r;
-          if (row < tc.row_end && col < a.N) {
-            const int orow = a.scatter ? a.sorted_scattered[row] : row;
-            *reinterpret_cast<u32x4*>(out + (size_t)orow * a.N + col) = val;
-          }
+          if (row < tc.row_end && col < a.N) *reinterpret_cast<u32x4*>(out + (size_t)orow_of[mb][it] * a.N + col) = val;
         }
       }
     }
@@ -931,19 +975,32 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     load_rows(c1, raw1);
     make_src(c0, raw0, src_cur);
     make_src(c1, raw1, src_next);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
   }
+  constexpr int AHEAD = PP ? NSTAGE - 1 : NSTAGE;  // slices in flight ahead of the one being consumed
+  static_assert(!PP || (BK == 32 && WN == 2 && STEPS == 2), "ping-pong shape");
 #pragma unroll
-  for (int st = 0; st < NSTAGE; ++st) dma_slice(src_cur, src_cur, false, st, st);
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm((NSTAGE - 1) * NLD, 0));
+  for (int st = 0; st < AHEAD; ++st) dma_slice(src_cur, src_cur, false, st, st);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm((AHEAD - 1) * NLD, 0));
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  read_frags(0, 0, 0);
+  if (!PP) read_frags(0, 0, 0);
 
   for (int i = 0;; ++i) {
-    // the ring runs on into the next tile: the last NSTAGE slices refill with its first NSTAGE
-    for (int kt = 0; kt < nk; ++kt) {
-      const bool from_next = kt >= nk - NSTAGE;
-      slice(src_cur, src_next, from_next, from_next ? kt + NSTAGE - nk : kt + NSTAGE);
+    // the ring runs on into the next tile: the last AHEAD slices refill with its first AHEAD
+    if (PP) {
+      // group wn == 1 runs one phase behind group wn == 0 inside a tile; both leave the tile together
+      if (wn == 1) __builtin_amdgcn_s_barrier();
+      for (int kt = 0; kt < nk; ++kt) {
+        const bool from_next = kt >= nk - AHEAD;
+        pp_slice(src_cur, src_next, from_next, from_next ? kt + AHEAD - nk : kt + AHEAD);
+      }
+      if (wn == 0) __builtin_amdgcn_s_barrier();
+    } else {
+      for (int kt = 0; kt < nk; ++kt) {
+        const bool from_next = kt >= nk - NSTAGE;
+        slice(src_cur, src_next, from_next, from_next ? kt + NSTAGE - nk : kt + NSTAGE);
+      }
     }
     const int t2 = tile_of(i + 2);
     TileCoord c2 = c1;
@@ -951,12 +1008,21 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     int raw2[NXLD];
     load_rows(c2, raw2);
     epilogue(c0);
-    if (t1 < 0) break;
+    if (t1 < 0) {
+      // The compiler folds this exit into the loop's back edge and then assumes, inside the slice loop, that
+      // the row-index loads above may still be in flight (nobody consumes them on this path): it would drain
+      // the DMA ring with vmcnt(0) at the top of every K slice.  Retiring them here keeps that path clean.
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+      break;
+    }
     c0 = c1;
     c1 = c2;
     t1 = t2;
     src_cur = src_next;
     make_src(c2, raw2, src_next);
+    // Retire every load the compiler knows about (row indices, epilogue traffic) here, once per tile:
+    // otherwise it re-checks them with vmcnt(0) inside the slice loop and drains the DMA ring there.
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));  // surplus DMA must not outlive the workgroup's LDS
 }
@@ -1031,12 +1097,12 @@ static int launch_dma(GemmArgs a, hipStream_t s) {
   return mi_launch_status();
 }
 
-template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool SCHED>
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool PP>
 static int launch_persistent(GemmArgs a, hipStream_t s) {
   constexpr int BN = GLU ? BNW / 2 : BNW;
   constexpr int NW = WM * WN;
   const size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T) + (size_t)NW * (NW > 4 ? 2048 : 4096) + (size_t)a.E * 8;
-  auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, BK, SCHED>;
+  auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, BK, PP>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;
@@ -1067,7 +1133,8 @@ static int launch_naive(GemmArgs a, hipStream_t s) {
 //   0 / 1 / 2  register-staged 256x256 / 128x128 / 32x256 (any K % 8 == 0)
 //   3          one thread per output element (any shape, any dtype)
 //   4          DMA-staged 128x128, one tile per workgroup (K % 32 == 0)
-//   5 / 6      persistent DMA-staged 256x256, 8 waves, 32-wide / 64-wide K slices
+//   5 / 6      persistent DMA-staged 256x256, 8 waves, 32-wide / 64-wide K slices, all waves in one phase
+//   7          persistent DMA-staged 256x256, 8 waves, 32-wide K slices, two wave groups in ping-pong
 template <typename T, bool GLU>
 static int dispatch_cfg(GemmArgs a, int cfg, hipStream_t s) {
   switch (cfg) {
@@ -1079,6 +1146,7 @@ static int dispatch_cfg(GemmArgs a, int cfg, hipStream_t s) {
     case 6:
       return persistent_ok(a) && a.K % 64 == 0 ? launch_persistent<T, 256, 256, 4, 2, GLU, 64, false>(a, s)
                                                : MI_MOE_EUNSUPPORTED;
+    case 7: return persistent_ok(a) ? launch_persistent<T, 256, 256, 4, 2, GLU, 32, true>(a, s) : MI_MOE_EUNSUPPORTED;
     default: return MI_MOE_EUNSUPPORTED;
   }
 }
@@ -1094,7 +1162,7 @@ static bool tiled_ok(const GemmArgs& a, int in_rows_bound, bool glu) {
 
 static int pick_cfg(const GemmArgs& a) {
   const long avg = a.E > 0 ? (long)a.L / a.E : a.L;  // rows per expert if the load were uniform
-  if (avg >= 192 && persistent_ok(a)) return a.K % 64 == 0 ? 6 : 5;
+  if (avg >= 192 && persistent_ok(a)) return 7;
   if (avg >= 512) return 0;
   if (avg >= 48) return a.K % 32 == 0 ? 4 : 1;
   return 2;

@@ -51,13 +51,13 @@ CASES = [
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,E,k,K,N", CASES)
 @pytest.mark.parametrize("mode", ["scatter2group", "group2scatter", "scatter2scatter", "group2group"])
-@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4, 5, 6, 7])
 def test_scattered_gemm(device, dtype, T, E, k, K, N, mode, cfg):
     if dtype == torch.float32 and cfg not in (-1, 3):
         pytest.skip("tiled configurations are 16-bit only")
     if cfg == 4 and K % 32:
         pytest.skip("the DMA-staged kernel needs K % 32 == 0")
-    if cfg in (5, 6) and (K % (64 if cfg == 6 else 32) or K < 128 or N % 8):
+    if cfg in (5, 6, 7) and (K % (64 if cfg == 6 else 32) or K < 128 or N % 8):
         pytest.skip("the persistent kernel needs K % 32 (64) == 0, K >= 128, N % 8 == 0")
     ops = _ops()
     g = torch.Generator().manual_seed(T * 3 + E + K + N)
@@ -76,13 +76,13 @@ def test_scattered_gemm(device, dtype, T, E, k, K, N, mode, cfg):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,E,k,H,I", [(15, 8, 8, 32, 128), (512, 8, 2, 256, 512), (333, 5, 2, 136, 100),
                                        (2048, 4, 2, 512, 256), (64, 64, 6, 256, 128)])
-@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4, 5, 6, 7])
 def test_up_swiglu(device, dtype, T, E, k, H, I, cfg):
     if dtype == torch.float32 and cfg not in (-1, 3):
         pytest.skip("tiled configurations are 16-bit only")
     if cfg == 4 and H % 32:
         pytest.skip("the DMA-staged kernel needs K % 32 == 0")
-    if cfg in (5, 6) and (H % (64 if cfg == 6 else 32) or H < 128 or I % 8):
+    if cfg in (5, 6, 7) and (H % (64 if cfg == 6 else 32) or H < 128 or I % 8):
         pytest.skip("the persistent kernel needs K % 32 (64) == 0, K >= 128, N % 8 == 0")
     ops = _ops()
     g = torch.Generator().manual_seed(T + H + I)
@@ -110,6 +110,44 @@ def test_gemm_identity_weights_permutes_rows(device):
     assert torch.equal(out2.cpu(), x.repeat_interleave(k, dim=0))
 
 
+@pytest.mark.parametrize("cfg", [2, 3, 5, 7])
+def test_gemm_bf16_rounding_is_nearest_even(device, cfg):
+    """The final fp32 -> bf16 rounding is round-to-nearest-even, bit for bit (ties, carries into the
+    exponent, overflow to inf, NaN): out = a + b where the fp32 sum is exact, so the only rounding in the
+    whole computation is the conversion of the result.  (fp32-denormal results are left out: what the
+    matrix cores do with denormal operands is not part of the contract.)"""
+    ops = _ops()
+    g = torch.Generator().manual_seed(11)
+    T, K, N = 8192, 128, 8
+    # a: random normal bf16 bit patterns with moderate exponents, b: a few binades (0..12) below a
+    a_bits = (torch.randint(0, 2, (T,), generator=g) << 15) | (torch.randint(100, 150, (T,), generator=g) << 7) \
+        | torch.randint(0, 128, (T,), generator=g)
+    shift = torch.randint(0, 13, (T,), generator=g)
+    b_bits = (torch.randint(0, 2, (T,), generator=g) << 15) | ((((a_bits >> 7) & 0xff) - shift) << 7) \
+        | torch.randint(0, 128, (T,), generator=g)
+    a = a_bits.to(torch.int16).view(torch.bfloat16)
+    b = b_bits.to(torch.int16).view(torch.bfloat16)
+    # hand-made rows: exact ties (to even, both directions), carry into the next binade, overflow, NaN, inf
+    special = [(1.0, 2.0 ** -8), (1.0 + 2.0 ** -7, 2.0 ** -8), (1.0, 2.0 ** -8 + 2.0 ** -15), (1.9921875, 2.0 ** -8),
+               (-1.0, -(2.0 ** -8)), (3.3895313892515355e38, 3.3895313892515355e38), (float("nan"), 1.0),
+               (float("inf"), 1.0), (float("-inf"), 1.0), (0.0, 0.0), (1.0, -1.0)]
+    for i, (u, v) in enumerate(special):
+        a[i], b[i] = u, v
+    x = torch.zeros(T, K, dtype=torch.bfloat16)
+    x[:, 0], x[:, 77] = a, b
+    w = torch.zeros(1, N, K, dtype=torch.bfloat16)
+    w[0, :, 0] = 1.0
+    w[0, :, 77] = 1.0
+    idx = torch.arange(T, dtype=torch.int32)
+    off = torch.tensor([T], dtype=torch.int32)
+    out = ops.scattered_gemm(x.to(device), w.to(device), 1, idx.to(device), off.to(device), False, False, cfg=cfg).cpu()
+    want = (a.float() + b.float()).to(torch.bfloat16)
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(out[:, 0]), nan)
+    for n in range(N):
+        assert torch.equal(out[~nan, n].view(torch.int16), want[~nan].view(torch.int16)), n
+
+
 def test_gemm_empty_experts_and_single_expert(device):
     ops = _ops()
     g = torch.Generator().manual_seed(3)
@@ -118,7 +156,7 @@ def test_gemm_empty_experts_and_single_expert(device):
     se, ss, off = oracle.sort_bin(sel, E)
     x = _rand((T, K), 1.0, torch.bfloat16, g)
     w = _rand((E, N, K), 0.05, torch.bfloat16, g)
-    for cfg in (0, 1, 2, 3, 4, 5, 6):
+    for cfg in (0, 1, 2, 3, 4, 5, 6, 7):
         out = ops.scattered_gemm(x.to(device), w.to(device), k, ss.to(device), off.to(device), False, False, cfg=cfg)
         ref = x.float() @ w[9].float().t()
         torch.testing.assert_close(out.cpu().float(), ref, rtol=2e-2, atol=2e-2)
