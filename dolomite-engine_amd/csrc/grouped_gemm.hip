@@ -24,6 +24,8 @@
 //     written to the other stage afterwards; one barrier per K-tile.
 #include "common.h"
 
+#include <type_traits>
+
 template <typename T> struct Mfma32;
 template <> struct Mfma32<bf16_t> {
   typedef bf16x8 vec;
@@ -35,6 +37,23 @@ template <> struct Mfma32<f16_t> {
   typedef f16x8 vec;
   static __device__ __forceinline__ f32x16 run(vec a, vec b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// 16x16x32: half the flops per instruction and the same rate, but a quarter of the accumulator traffic
+// per flop.  Under the chip's power limit (random operands) it sustains about 30 % more throughput than
+// 32x32x16, so the persistent ping-pong kernel uses it.
+template <typename T> struct Mfma16;
+template <> struct Mfma16<bf16_t> {
+  typedef bf16x8 vec;
+  static __device__ __forceinline__ f32x4 run(vec a, vec b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16<f16_t> {
+  typedef f16x8 vec;
+  static __device__ __forceinline__ f32x4 run(vec a, vec b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
 };
 
@@ -660,17 +679,20 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
   constexpr int EPI_COLS = NW > 4 ? 32 : 64; // per-wave epilogue scratch: 32 rows x EPI_COLS columns
   constexpr int EPI_BYTES = 32 * EPI_COLS * 2;
-  constexpr int EPI_OB = EPI_COLS / 32;      // 32-column blocks per epilogue pass
   constexpr int EPI_CPR = EPI_COLS / 8;      // 16-byte chunks per scratch row
   constexpr int NLD = ROWS / RPI / NW;       // DMA instructions per wave per K slice
   constexpr int NXLD = BM / RPI / NW;        // ... of which activation rows (the first NXLD)
   constexpr int BN = GLU ? BNW / 2 : BNW;
   constexpr int WTM = BM / WM, WTN = BNW / WN;
-  constexpr int MB = WTM / 32, NB = WTN / 32;
+  // matrix instruction: 32x32x16 (two k steps per 32-wide slice), or with PP 16x16x32 (one step per slice)
+  constexpr int MT = PP ? 16 : 32;           // edge of one accumulator block
+  constexpr int ACC_GROUPS = PP ? 1 : 4;     // 4-register groups per accumulator block
+  constexpr int MB = WTM / MT, NB = WTN / MT;
   constexpr int OB = GLU ? NB / 2 : NB;      // output column blocks per wave
-  constexpr int NMFMA = MB * NB;
+  constexpr int EPI_MB = 32 / MT;            // accumulator row blocks per 32-row epilogue pass
+  constexpr int EPI_NB = EPI_COLS / MT;      // accumulator column blocks per epilogue pass
   static_assert(BM % (16 * NW) == 0 && BNW % (16 * NW) == 0 && NW % 2 == 0, "tile/wave shape");
-  static_assert(OB % EPI_OB == 0, "epilogue pass shape");
+  static_assert(OB % EPI_NB == 0 && MB % EPI_MB == 0, "epilogue pass shape");
   static_assert((NSTAGE - 1) * NLD <= 63, "vmcnt range");
   typedef typename Mfma32<T>::vec frag_t;
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -717,25 +739,39 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     const int t = xcd * per + local;
     return (local < per && t < total) ? t : -1;
   };
-  // tile id -> coordinates, from the LDS table (wave-uniform result)
+  // tile id -> coordinates, from the LDS table (wave-uniform result).  An expert's tiles are numbered band
+  // by band: a band is up to 8 column tiles wide and runs over all of the expert's row tiles, row tile
+  // slowest.  The 32 workgroups of an XCD, which take 32 consecutive tiles at a time, then cover about
+  // 4 row tiles x 8 column tiles: 12 operand slabs for 32 tiles, and each weight slab is fetched once per
+  // band instead of once per row tile (with many column tiles -- intermediate 14336 -- a plain row-major
+  // order re-streams all of an expert's weights from HBM for every row tile).  Up to 8 column tiles the band
+  // is the whole row, so that complete output rows are written at about the same time.
+  const int tile_band = a.n_tiles < 8 ? a.n_tiles : 8;
   auto locate = [&](int tile, TileCoord& tc) {
-    const int mt = tile / a.n_tiles;
-    tc.nt = tile - mt * a.n_tiles;
+    const int q = tile / a.n_tiles;  // experts own contiguous tile ranges: (row tiles before) * n_tiles
     for (int e0 = 0; e0 < a.E; e0 += 64) {
       const int e = e0 + lane;
       const int incl = e < a.E ? etab[2 * e] : 0x7fffffff;
-      const uint64_t hit = __ballot(incl > mt);
+      const uint64_t hit = __ballot(incl > q);
       if (hit) {
         const int ex = e0 + __ffsll((long long)hit) - 1;
         const int first_tile = ex > 0 ? etab[2 * (ex - 1)] : 0;
         const int prev = ex > 0 ? etab[2 * (ex - 1) + 1] : 0;
+        const int row_tiles = etab[2 * ex] - first_tile;
+        const int local = tile - first_tile * a.n_tiles;
+        const int band = local / (row_tiles * tile_band);
+        const int rem = local - band * row_tiles * tile_band;
+        const int left = a.n_tiles - band * tile_band;
+        const int width = left < tile_band ? left : tile_band;
+        const int mt = rem / width;
         tc.expert = ex;
-        tc.row_begin = prev + (mt - first_tile) * BM;
+        tc.nt = band * tile_band + rem - mt * width;
+        tc.row_begin = prev + mt * BM;
         tc.row_end = etab[2 * ex + 1];
         return;
       }
     }
-    tc.expert = 0; tc.row_begin = 0; tc.row_end = 1;  // unreachable for a valid tile id
+    tc.expert = 0; tc.nt = 0; tc.row_begin = 0; tc.row_end = 1;  // unreachable for a valid tile id
   };
 
   // ---- DMA sources -----------------------------------------------------------------------------------
@@ -802,28 +838,31 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   };
 
   // ---- fragment reads ----------------------------------------------------------------------------------
-  const int frow = lane & 31, fhalf = lane >> 5;
+  // lane -> (row of its MT-row block, k chunk): 32x32x16 takes k = 8 * (lane / 32) + [0, 8) of a 16-wide step,
+  // 16x16x32 takes k = 8 * (lane / 16) + [0, 8) of the whole 32-wide slice
+  const int frow = lane % MT, fhalf = lane / MT;
   const int fswz = BK == 32 ? ((frow >> 2) & 3) : ((frow & 7) ^ ((frow >> 3) & 1));
   int frag_x_off[MB], frag_w_off[NB];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) frag_x_off[mb] = (wm * WTM + mb * 32 + frow) * (BK * 2);
+  for (int mb = 0; mb < MB; ++mb) frag_x_off[mb] = (wm * WTM + mb * MT + frow) * (BK * 2);
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     int r;
     if (GLU) {
       constexpr int HB = NB / 2;
       int h = nb >= HB;
-      r = h * BN + wn * (WTN / 2) + (h ? nb - HB : nb) * 32 + frow;
+      r = h * BN + wn * (WTN / 2) + (h ? nb - HB : nb) * MT + frow;
     } else {
-      r = wn * WTN + nb * 32 + frow;
+      r = wn * WTN + nb * MT + frow;
     }
     frag_w_off[nb] = (BM + r) * (BK * 2);
   }
   int chunk_byte[STEPS];
 #pragma unroll
-  for (int kk = 0; kk < STEPS; ++kk) chunk_byte[kk] = ((2 * kk + fhalf) ^ fswz) * 16;
+  for (int kk = 0; kk < STEPS; ++kk) chunk_byte[kk] = (((PP ? 0 : 2 * kk) + fhalf) ^ fswz) * 16;
 
-  frag_t xf[2][MB], wf[2][NB];
+  constexpr int NBUF = PP ? 1 : 2;
+  frag_t xf[NBUF][MB], wf[NBUF][NB];
   auto read_frags = [&](int stage, int kk, int buf) {
     const unsigned char* s = smem_raw + stage * STAGE_BYTES + chunk_byte[kk];
 #pragma unroll
@@ -834,19 +873,25 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
       xf[buf][mb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_x_off[mb]));
   };
 
-  f32x16 acc[NB][MB];
+  // accumulator block (nb, mb): register 4 * g + i of a lane is output column MT * nb + 8 * g + 4 * fhalf + i
+  // (weight row) of token row MT * mb + frow
+  typedef typename std::conditional<PP, f32x4, f32x16>::type acc_t;
+  acc_t acc[NB][MB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[nb][mb][i] = 0.f;
+      for (int i = 0; i < 4 * ACC_GROUPS; ++i) acc[nb][mb][i] = 0.f;
 
   auto mfma_step = [&](int buf) {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = Mfma32<T>::run(wf[buf][nb], xf[buf][mb], acc[nb][mb]);
+      for (int mb = 0; mb < MB; ++mb) {
+        if constexpr (PP) acc[nb][mb] = Mfma16<T>::run(wf[buf][nb], xf[buf][mb], acc[nb][mb]);
+        else acc[nb][mb] = Mfma32<T>::run(wf[buf][nb], xf[buf][mb], acc[nb][mb]);
+      }
   };
 
   int g = 0;  // running K-slice count; slice g lives in ring stage g % NSTAGE
@@ -872,7 +917,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   };
   // Ping-pong form of one K slice (PP; BK = 32, four stages).  The waves with wn == 0 and those with
   // wn == 1 -- one of each per SIMD -- run this same code one phase apart (see the tile loop): while one group
-  // issues its 2 * NMFMA matrix instructions back to back out of registers, the other reads its fragments of the
+  // issues its NB * MB matrix instructions back to back out of registers, the other reads its fragments of the
   // slice from LDS and issues its share of the DMA for slice g + 3 into the stage both groups have finished
   // reading.  Every phase ends in a workgroup barrier; at each barrier one group has just issued its last MFMA
   // and the other has its operands in registers, so the matrix pipe of the SIMD never waits for LDS, DMA or the
@@ -880,7 +925,6 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   auto pp_slice = [&](const TileSrc& tcur, const TileSrc& tnext, bool from_next, int kload) {
     const int cur = g & (NSTAGE - 1), fill = (g + NSTAGE - 1) & (NSTAGE - 1);
     read_frags(cur, 0, 0);
-    read_frags(cur, 1, 1);
     dma_slice(tcur, tnext, from_next, kload, fill);
     asm volatile("" ::: "memory");
     // own DMA of slice g + 1 has landed (slices g + 2 and g + 3 stay in flight); fragments are in registers
@@ -888,8 +932,9 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
+    // (Signalling the second barrier a few matrix instructions early, so that they cover its release
+    // latency, measured slower: the group's next memory phase then starts late and becomes the long one.)
     mfma_step(0);
-    mfma_step(1);
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -901,43 +946,51 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   unsigned char* scratch = smem_raw + RING_BYTES + wave * EPI_BYTES;
   auto epilogue = [&](const TileCoord& tc) {
     // scratch row r keeps its EPI_CPR 16-byte chunks at slots chunk ^ swz(r): the 8-byte writes of a
-    // wave (32 rows, one chunk) and the 16-byte read-back both spread over all banks
+    // wave and the 16-byte read-back both spread over all banks
     auto swz = [](int r) { return EPI_CPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3); };
     constexpr int RPP = 64 / EPI_CPR;  // rows per read-back pass
+    constexpr int MP = MB / EPI_MB;    // 32-row passes over the wave's token rows
     // destination rows of everything this lane will store, fetched up front: one memory latency per tile
     // instead of one per store
-    int orow_of[MB][32 / RPP];
+    int orow_of[MP][32 / RPP];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+    for (int mp = 0; mp < MP; ++mp)
 #pragma unroll
       for (int it = 0; it < 32 / RPP; ++it) {
-        const int row = tc.row_begin + wm * WTM + mb * 32 + it * RPP + lane / EPI_CPR;
-        orow_of[mb][it] = (a.scatter && row < tc.row_end) ? a.sorted_scattered[row] : row;
+        const int row = tc.row_begin + wm * WTM + mp * 32 + it * RPP + lane / EPI_CPR;
+        orow_of[mp][it] = (a.scatter && row < tc.row_end) ? a.sorted_scattered[row] : row;
       }
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
+    for (int mp = 0; mp < MP; ++mp) {
 #pragma unroll
-      for (int og = 0; og < OB / EPI_OB; ++og) {
-        // write the 32 x EPI_COLS block: lane holds row frow, columns ob*32 + g*8 + fhalf*4 + [0,4)
+      for (int og = 0; og < OB / EPI_NB; ++og) {
+        // write the 32 x EPI_COLS block: a lane holds, per accumulator block, token row frow and the four
+        // output columns 8 * g + 4 * fhalf + [0, 4) of each group g
 #pragma unroll
-        for (int ob = 0; ob < EPI_OB; ++ob) {
-          const int nb = og * EPI_OB + ob;
+        for (int mbb = 0; mbb < EPI_MB; ++mbb) {
+          const int mb = mp * EPI_MB + mbb;
+          const int srow = mbb * MT + frow;
 #pragma unroll
-          for (int gq = 0; gq < 4; ++gq) {
-            float v[4];
+          for (int ob = 0; ob < EPI_NB; ++ob) {
+            const int nb = og * EPI_NB + ob;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              if (GLU) {
-                const float up = acc[nb][mb][gq * 4 + i];
-                const float gt = acc[nb + NB / 2][mb][gq * 4 + i];
-                v[i] = up * gt * __builtin_amdgcn_rcpf(1.0f + __expf(-gt));
-              } else {
-                v[i] = acc[nb][mb][gq * 4 + i];
+            for (int gq = 0; gq < ACC_GROUPS; ++gq) {
+              float v[4];
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                if (GLU) {
+                  const float up = acc[nb][mb][gq * 4 + i];
+                  const float gt = acc[nb + NB / 2][mb][gq * 4 + i];
+                  v[i] = up * gt * __builtin_amdgcn_rcpf(1.0f + __expf(-gt));
+                } else {
+                  v[i] = acc[nb][mb][gq * 4 + i];
+                }
               }
+              const int colp = ob * MT + gq * 8 + fhalf * 4;  // column inside the pass
+              const u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+              *reinterpret_cast<u32x2*>(scratch + srow * (EPI_COLS * 2) + (((colp >> 3) ^ swz(srow)) * 16) +
+                                        ((colp >> 2) & 1) * 8) = p;
             }
-            const int chunk = ob * 4 + gq;
-            const u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
-            *reinterpret_cast<u32x2*>(scratch + frow * (EPI_COLS * 2) + ((chunk ^ swz(frow)) * 16) + fhalf * 8) = p;
           }
         }
         // read back: lane -> row it*RPP + lane/EPI_CPR, 16-byte chunk lane%EPI_CPR
@@ -947,8 +1000,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
         for (int it = 0; it < 32 / RPP; ++it) {
           const int r = it * RPP + lane / EPI_CPR;
           const u32x4 val = *reinterpret_cast<const u32x4*>(scratch + r * (EPI_COLS * 2) + ((cchunk ^ swz(r)) * 16));
-          const int row = tc.row_begin + wm * WTM + mb * 32 + r;
-          if (row < tc.row_end && col < a.N) *reinterpret_cast<u32x4*>(out + (size_t)orow_of[mb][it] * a.N + col) = val;
+          const int row = tc.row_begin + wm * WTM + mp * 32 + r;
+          if (row < tc.row_end && col < a.N) *reinterpret_cast<u32x4*>(out + (size_t)orow_of[mp][it] * a.N + col) = val;
         }
       }
     }
@@ -957,7 +1010,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[nb][mb][i] = 0.f;
+        for (int i = 0; i < 4 * ACC_GROUPS; ++i) acc[nb][mb][i] = 0.f;
   };
 
   // ---- tile loop -------------------------------------------------------------------------------------------
@@ -978,7 +1031,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
   }
   constexpr int AHEAD = PP ? NSTAGE - 1 : NSTAGE;  // slices in flight ahead of the one being consumed
-  static_assert(!PP || (BK == 32 && WN == 2 && STEPS == 2), "ping-pong shape");
+  static_assert(!PP || (BK == 32 && WN == 2), "ping-pong shape");
 #pragma unroll
   for (int st = 0; st < AHEAD; ++st) dma_slice(src_cur, src_cur, false, st, st);
   __builtin_amdgcn_s_waitcnt(waitcnt_imm((AHEAD - 1) * NLD, 0));
