@@ -37,30 +37,48 @@ template <typename T> struct Chunk16 {
 template <> struct Chunk<bf16_t> : Chunk16<bf16_t> {};
 template <> struct Chunk<f16_t> : Chunk16<f16_t> {};
 
-template <typename T>
+// A workgroup walks whole token rows (grid-stride over tokens, threads over the row's 16-byte chunks): no
+// division per element, the k gates of a row are wave-uniform, and with K known at compile time all k loads
+// of a chunk are in flight together.  K == 0 is the run-time-k version.
+template <typename T, int K>
 __global__ __launch_bounds__(256) void combine_vec_kernel(const T* __restrict__ o, const T* __restrict__ gates,
-                                                          T* __restrict__ y, int Trows, int k, int H) {
+                                                          T* __restrict__ y, int Trows, int k_rt, int H) {
   constexpr int V = Chunk<T>::N;
+  const int k = K > 0 ? K : k_rt;
   const int cpr = H / V;  // chunks per row
-  const long total = (long)Trows * cpr;
-  for (long id = (long)blockIdx.x * 256 + threadIdx.x; id < total; id += (long)gridDim.x * 256) {
-    const int t = (int)(id / cpr);
-    const int c = (int)(id - (long)t * cpr);
-    float acc[V];
-#pragma unroll
-    for (int i = 0; i < V; ++i) acc[i] = 0.f;
-    const T* src = o + ((size_t)t * k) * H + (size_t)c * V;
+  for (int t = blockIdx.x; t < Trows; t += gridDim.x) {
     const T* g = gates + (size_t)t * k;
-#pragma unroll 4
-    for (int j = 0; j < k; ++j) {
-      const float gj = Elt<T>::load(g + j);
-      const u32x4 v = *reinterpret_cast<const u32x4*>(src + (size_t)j * H);
-      float f[V];
-      Chunk<T>::unpack(v, f);
+    const T* row = o + ((size_t)t * k) * H;
+    for (int c = threadIdx.x; c < cpr; c += blockDim.x) {
+      float acc[V];
 #pragma unroll
-      for (int i = 0; i < V; ++i) acc[i] = fmaf(gj, f[i], acc[i]);
+      for (int i = 0; i < V; ++i) acc[i] = 0.f;
+      const T* src = row + (size_t)c * V;
+      if (K > 0) {
+        u32x4 v[K > 0 ? K : 1];
+#pragma unroll
+        for (int j = 0; j < K; ++j) v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + (size_t)j * H));
+#pragma unroll
+        for (int j = 0; j < K; ++j) {
+          const float gj = Elt<T>::load(g + j);
+          float f[V];
+          Chunk<T>::unpack(v[j], f);
+#pragma unroll
+          for (int i = 0; i < V; ++i) acc[i] = fmaf(gj, f[i], acc[i]);
+        }
+      } else {
+#pragma unroll 4
+        for (int j = 0; j < k; ++j) {
+          const float gj = Elt<T>::load(g + j);
+          const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + (size_t)j * H));
+          float f[V];
+          Chunk<T>::unpack(v, f);
+#pragma unroll
+          for (int i = 0; i < V; ++i) acc[i] = fmaf(gj, f[i], acc[i]);
+        }
+      }
+      __builtin_nontemporal_store(Chunk<T>::pack(acc), reinterpret_cast<u32x4*>(y + (size_t)t * H + (size_t)c * V));
     }
-    *reinterpret_cast<u32x4*>(y + (size_t)t * H + (size_t)c * V) = Chunk<T>::pack(acc);
   }
 }
 
@@ -78,19 +96,37 @@ __global__ __launch_bounds__(256) void combine_scalar_kernel(const T* __restrict
   }
 }
 
+template <typename T, int K>
+static void launch_combine_vec(const void* o, const void* gates, void* y, int T_, int k, int H, hipStream_t s) {
+  constexpr int V = Chunk<T>::N;
+  const int cpr = H / V;
+  int threads = cpr >= 256 ? 256 : (cpr + 63) / 64 * 64;  // whole waves, at most one pass over short rows
+  long blocks = T_;
+  if (blocks > 256L * 32) blocks = 256L * 32;
+  hipLaunchKernelGGL((combine_vec_kernel<T, K>), dim3((unsigned)blocks), dim3(threads), 0, s,
+                     static_cast<const T*>(o), static_cast<const T*>(gates), static_cast<T*>(y), T_, k, H);
+}
+
 template <typename T>
 static int launch_combine(const void* o, const void* gates, void* y, int T_, int k, int H, hipStream_t s) {
   constexpr int V = Chunk<T>::N;
   const bool vec = (H % V == 0) && mi_aligned(o, 16) && mi_aligned(y, 16);
-  const long work = vec ? (long)T_ * (H / V) : (long)T_ * H;
-  long blocks = (work + 255) / 256;
-  if (blocks > 256L * 64) blocks = 256L * 64;
-  if (vec)
-    hipLaunchKernelGGL((combine_vec_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const T*>(o),
-                       static_cast<const T*>(gates), static_cast<T*>(y), T_, k, H);
-  else
+  if (vec) {
+    switch (k) {
+      case 1: launch_combine_vec<T, 1>(o, gates, y, T_, k, H, s); break;
+      case 2: launch_combine_vec<T, 2>(o, gates, y, T_, k, H, s); break;
+      case 4: launch_combine_vec<T, 4>(o, gates, y, T_, k, H, s); break;
+      case 6: launch_combine_vec<T, 6>(o, gates, y, T_, k, H, s); break;
+      case 8: launch_combine_vec<T, 8>(o, gates, y, T_, k, H, s); break;
+      default: launch_combine_vec<T, 0>(o, gates, y, T_, k, H, s); break;
+    }
+  } else {
+    const long work = (long)T_ * H;
+    long blocks = (work + 255) / 256;
+    if (blocks > 256L * 64) blocks = 256L * 64;
     hipLaunchKernelGGL((combine_scalar_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s,
                        static_cast<const T*>(o), static_cast<const T*>(gates), static_cast<T*>(y), T_, k, H);
+  }
   return mi_launch_status();
 }
 

@@ -243,6 +243,137 @@ __global__ __launch_bounds__(1024) void router_fused_small_kernel(const T* __res
   }
 }
 
+// Few tokens, K split across workgroups.  One workgroup reads at most 26 bytes per clock, and a 16-token group
+// needs all of the gate weights (E x H): four workgroups pulling 640 KB each take 20+ us for a 64-token batch.
+// Here workgroup (tg, ks) takes K range ks of token group tg (four waves, one 64-wide K step each per
+// round) and writes its 16 x 64 partial logits, as raw accumulator registers, to the workspace; a second
+// launch adds the partials in a fixed order (the logits do not depend on scheduling) and runs the epilogue.
+#define ROUTER_SPLIT_WAVES 4
+template <typename T>
+__global__ __launch_bounds__(ROUTER_SPLIT_WAVES * 64) void router_splitk_partial_kernel(
+    const T* __restrict__ x, const T* __restrict__ gw, int Trows, int H, int E, int steps_per_split,
+    f32x4* __restrict__ partial) {
+  typedef typename RMfma<T>::vec frag_t;
+  __shared__ f32x4 red[ROUTER_SPLIT_WAVES][4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int tg = blockIdx.x, ks = blockIdx.y;
+  int t = tg * 16 + r;
+  if (t > Trows - 1) t = Trows - 1;
+  const T* xrow = x + (size_t)t * H;
+  const T* wrow[4];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) {
+    int e = eb * 16 + r;
+    if (e > E - 1) e = E - 1;
+    wrow[eb] = gw + (size_t)e * H;
+  }
+  f32x4 acc[4];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) acc[eb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const int step0 = ks * steps_per_split;
+  for (int st = wave; st < steps_per_split; st += ROUTER_SPLIT_WAVES) {
+    const int kpos = (step0 + st) * 64 + q * 16;
+    const bool valid = kpos < H;  // the MFMA runs on all lanes: out-of-range k contributes zeros
+    u32x4 x0 = {0u, 0u, 0u, 0u}, x1 = {0u, 0u, 0u, 0u};
+    u32x4 w0[4], w1[4];
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) w0[eb] = w1[eb] = (u32x4){0u, 0u, 0u, 0u};
+    if (valid) {
+      x0 = *reinterpret_cast<const u32x4*>(xrow + kpos);
+      x1 = *reinterpret_cast<const u32x4*>(xrow + kpos + 8);
+#pragma unroll
+      for (int eb = 0; eb < 4; ++eb) {
+        w0[eb] = *reinterpret_cast<const u32x4*>(wrow[eb] + kpos);
+        w1[eb] = *reinterpret_cast<const u32x4*>(wrow[eb] + kpos + 8);
+      }
+    }
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) {
+      acc[eb] = RMfma<T>::run(__builtin_bit_cast(frag_t, w0[eb]), __builtin_bit_cast(frag_t, x0), acc[eb]);
+      acc[eb] = RMfma<T>::run(__builtin_bit_cast(frag_t, w1[eb]), __builtin_bit_cast(frag_t, x1), acc[eb]);
+    }
+  }
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) red[wave][eb][lane] = acc[eb];
+  __syncthreads();
+  if (wave == 0) {
+    f32x4* dst = partial + ((size_t)ks * gridDim.x + tg) * 4 * 64;
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) {
+      f32x4 sum = red[0][eb][lane];
+#pragma unroll
+      for (int w = 1; w < ROUTER_SPLIT_WAVES; ++w) sum += red[w][eb][lane];
+      dst[eb * 64 + lane] = sum;
+    }
+  }
+}
+
+// Four waves per token group: wave w adds splits w, w + 4, ... (all of its loads in flight at once), wave 0 adds
+// the four sums in wave order and runs the epilogue.  The order of additions is fixed by the launch shape alone.
+template <typename T>
+__global__ __launch_bounds__(256) void router_splitk_finish_kernel(const f32x4* __restrict__ partial, int splits,
+                                                                   const float* __restrict__ bias, int Trows, int E, int k,
+                                                                   T* __restrict__ logits_out, T* __restrict__ gates,
+                                                                   int32_t* __restrict__ idx) {
+  __shared__ f32x4 red[4][4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int tg = blockIdx.x;
+  const int t = tg * 16 + r;
+  f32x4 acc[4];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) acc[eb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int ks = wave; ks < splits; ks += 4) {
+    const f32x4* src = partial + ((size_t)ks * gridDim.x + tg) * 4 * 64;
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) acc[eb] += src[eb * 64 + lane];
+  }
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) red[wave][eb][lane] = acc[eb];
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) {
+    f32x4 sum = red[0][eb][lane];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) sum += red[w][eb][lane];
+    acc[eb] = sum;
+  }
+  router_epilogue<T>(acc, t, t < Trows, q, bias, E, k, logits_out, gates, idx);
+}
+
+// K splits for the few-token path: one 64-wide K step per wave and round, enough workgroups to occupy the chip
+static int router_splits(int T_, int H) {
+  const int steps = mi_ceil_div(H, 64);
+  int splits = mi_ceil_div(steps, ROUTER_SPLIT_WAVES);
+  const int groups = mi_ceil_div(T_, 16);
+  while (splits > 1 && (long)splits * groups > 1024) splits = (splits + 1) / 2;
+  return splits;
+}
+
+static size_t router_ws_bytes(int T_, int H) {
+  if (T_ <= 0 || T_ > 1024) return 0;
+  return (size_t)router_splits(T_, H) * mi_ceil_div(T_, 16) * 4 * 64 * sizeof(f32x4);
+}
+
+template <typename T>
+static int launch_router_splitk(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
+                                void* logits_out, void* gates, int32_t* idx, void* ws, hipStream_t s) {
+  const int splits = router_splits(T_, H);
+  const int steps_per_split = mi_ceil_div(mi_ceil_div(H, 64), splits);
+  const int groups = mi_ceil_div(T_, 16);
+  hipLaunchKernelGGL((router_splitk_partial_kernel<T>), dim3(groups, splits), dim3(ROUTER_SPLIT_WAVES * 64), 0, s,
+                     static_cast<const T*>(x), static_cast<const T*>(gw), T_, H, E, steps_per_split,
+                     static_cast<f32x4*>(ws));
+  int rc = mi_launch_status();
+  if (rc != MI_MOE_OK) return rc;
+  hipLaunchKernelGGL((router_splitk_finish_kernel<T>), dim3(groups), dim3(256), 0, s, static_cast<const f32x4*>(ws),
+                     splits, bias, T_, E, k, static_cast<T*>(logits_out), static_cast<T*>(gates), idx);
+  return mi_launch_status();
+}
+
 template <typename T>
 static int launch_router(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
                          void* logits_out, void* gates, int32_t* idx, hipStream_t s) {
@@ -260,9 +391,14 @@ static int launch_router(const void* x, const void* gw, const float* bias, int T
   return mi_launch_status();
 }
 
+extern "C" size_t mi_moe_router_fused_workspace_bytes(int T, int H, int E) {
+  (void)E;
+  return (T < 0 || H < 1) ? 0 : router_ws_bytes(T, H);
+}
+
 extern "C" int mi_moe_router_fused(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,
-                                   int dtype, void* logits_out, void* gates_out, int32_t* idx_out,
-                                   mi_moe_stream_t stream) {
+                                   int dtype, void* logits_out, void* gates_out, int32_t* idx_out, void* ws,
+                                   size_t ws_bytes, mi_moe_stream_t stream) {
   if (T < 0 || H < 1 || E < 1 || k < 1 || k > E) return MI_MOE_ESHAPE;
   if (E > 64 || k > ROUTER_KMAX || H % 16 != 0) return MI_MOE_EUNSUPPORTED;
   if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
@@ -270,6 +406,14 @@ extern "C" int mi_moe_router_fused(const void* x, const void* gate_w, const floa
   if (!x || !gate_w || !gates_out || !idx_out) return MI_MOE_ENULL;
   if (!mi_aligned(x, 16) || !mi_aligned(gate_w, 16)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t need = router_ws_bytes(T, H);
+  if (ws != nullptr && need > 0) {  // few tokens and a workspace: K split across workgroups
+    if (ws_bytes < need) return MI_MOE_EWORKSPACE;
+    if (!mi_aligned(ws, 16)) return MI_MOE_EALIGN;
+    if (dtype == MI_MOE_BF16)
+      return launch_router_splitk<bf16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, ws, s);
+    return launch_router_splitk<f16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, ws, s);
+  }
   if (dtype == MI_MOE_BF16) return launch_router<bf16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, s);
   return launch_router<f16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, s);
 }

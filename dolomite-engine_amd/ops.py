@@ -123,9 +123,10 @@ def router_fused_supported(x: torch.Tensor, num_experts: int, k: int) -> bool:
 
 
 def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch.Tensor | None = None,
-                 return_logits: bool = False):
+                 return_logits: bool = False, split_k: bool = True):
     """logits = x @ gate_weight^T (+bias) in x.dtype, top-k, softmax: one pass over x.
 
+    ``split_k=False`` withholds the workspace, i.e. forces the single-launch kernel for few tokens too.
     Returns (logits or None, gates (T,k), experts (T,k) int32)."""
     _dev(x, gate_weight, bias)
     _no_grad(x, gate_weight)
@@ -140,9 +141,13 @@ def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch
     logits = torch.empty((T, E), dtype=x.dtype, device=x.device) if return_logits else None
     gates = torch.empty((T, k), dtype=x.dtype, device=x.device)
     idx = torch.empty((T, k), dtype=torch.int32, device=x.device)
+    lib = _lib.load()
+    # non-zero for few tokens: K split over the chip
+    ws_bytes = lib.mi_moe_router_fused_workspace_bytes(T, H, E) if split_k else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
     with _stage("router_fused"):
-        check(_lib.load().mi_moe_router_fused(_ptr(x), _ptr(gate_weight), _ptr(bias), T, H, E, k, _code(x.dtype),
-                                             _ptr(logits), _ptr(gates), _ptr(idx), _stream()))
+        check(lib.mi_moe_router_fused(_ptr(x), _ptr(gate_weight), _ptr(bias), T, H, E, k, _code(x.dtype),
+                                     _ptr(logits), _ptr(gates), _ptr(idx), _ptr(ws), ws_bytes, _stream()))
     return logits, gates, idx
 
 

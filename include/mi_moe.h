@@ -71,10 +71,15 @@ int mi_moe_router_topk_softmax(const void* logits, int T, int E, int k, int dtyp
  *   x (T, H), gate_w (E, H) of `dtype` (F16 / BF16), H % 8 == 0, E <= 64
  *   bias       (E,) fp32 or NULL
  *   logits_out (T, E) of `dtype` or NULL (only the training-time aux loss reads it)
+ *   ws / ws_bytes  optional scratch, 16-byte aligned.  With at least
+ *                  mi_moe_router_fused_workspace_bytes(T, H, E) bytes (non-zero for T <= 1024) the
+ *                  contraction is split over many workgroups and finished by a second small launch -- a few
+ *                  tokens alone cannot keep more than T/16 compute units busy; with NULL one launch does it all.
  */
+size_t mi_moe_router_fused_workspace_bytes(int T, int H, int E);
 int mi_moe_router_fused(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,
-                        int dtype, void* logits_out, void* gates_out, int32_t* idx_out,
-                        mi_moe_stream_t stream);
+                        int dtype, void* logits_out, void* gates_out, int32_t* idx_out, void* ws,
+                        size_t ws_bytes, mi_moe_stream_t stream);
 
 /*
  * Histogram of expert ids.

@@ -68,8 +68,10 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_router_topk_softmax(None, 4, 8, 9, _lib.BF16, None, None, None) == E_SHAPE  # k > E
     assert lib.mi_moe_router_topk_softmax(None, 4, 8, 2, _lib.BF16, None, None, None) == E_NULL
     assert lib.mi_moe_router_topk_softmax(None, 0, 8, 2, _lib.BF16, None, None, None) == 0  # empty input
-    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 128, 2, _lib.BF16, None, None, None, None) == E_UNSUP
-    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 8, 2, _lib.F32, None, None, None, None) == E_DTYPE
+    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 128, 2, _lib.BF16, None, None, None, None, 0, None) == E_UNSUP
+    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 8, 2, _lib.F32, None, None, None, None, 0, None) == E_DTYPE
+    assert lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) > 0
+    assert lib.mi_moe_router_fused_workspace_bytes(32768, 1536, 40) == 0
     assert lib.mi_moe_count(None, -1, 8, None, None) == E_SHAPE
     assert lib.mi_moe_sort_bin(None, 4, 2, 0, None, None, None, None, 0, None) == E_SHAPE
     assert lib.mi_moe_sort_bin(None, 4, 2, 8, None, None, None, None, 0, None) == E_NULL

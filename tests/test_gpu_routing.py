@@ -128,3 +128,12 @@ def test_router_fused(device, dtype, T, H, E, k, bias):
     # (3) without materialising the logits the result is the same
     _, gates2, idx2 = ops.router_fused(x.to(device), w.to(device), k, bias=None if b is None else b.to(device))
     assert torch.equal(idx2, idx) and torch.equal(gates2, gates)
+    # (4) the single-launch kernel (no workspace) sums K in another order: same contract on its own logits
+    logits3, gates3, idx3 = ops.router_fused(x.to(device), w.to(device), k, bias=None if b is None else b.to(device),
+                                             return_logits=True, split_k=False)
+    torch.testing.assert_close(logits3.cpu().float(), ref_logits.float(),
+                               rtol=1.6e-2 if dtype == torch.bfloat16 else 2e-3, atol=1e-3)
+    vals3, ref_idx3 = oracle.topk_canonical(logits3.cpu(), k)
+    assert torch.equal(idx3.cpu().long(), ref_idx3)
+    ulp3 = (gates3.cpu().view(torch.int16).int() - oracle.softmax_topk(vals3, dtype).view(torch.int16).int()).abs().max()
+    assert ulp3 <= 1
