@@ -677,7 +677,11 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   constexpr int ROWS = BM + BNW;
   constexpr int STAGE_BYTES = ROWS * BK * 2;
   constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
-  constexpr int EPI_COLS = NW > 4 ? 32 : 64; // per-wave epilogue scratch: 32 rows x EPI_COLS columns
+  // per-wave epilogue scratch: 32 rows x EPI_COLS columns.  64 columns make every store a run of whole
+  // 128-byte lines per row (measured: 64-byte pieces write at 4.4-4.6 TB/s chip-wide, 128-byte ones at
+  // 5.0-5.3).  The ping-pong kernel has a free ring stage to put it in; the others carve it out of what is
+  // left of LDS next to a full ring.
+  constexpr int EPI_COLS = (PP || NW <= 4) ? 64 : 32;
   constexpr int EPI_BYTES = 32 * EPI_COLS * 2;
   constexpr int EPI_CPR = EPI_COLS / 8;      // 16-byte chunks per scratch row
   constexpr int NLD = ROWS / RPI / NW;       // DMA instructions per wave per K slice
@@ -699,8 +703,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  // [ring: 4 stages][epilogue scratch: NW x 4 KiB][expert table: E x (tiles inclusive, row end)]
-  int* etab = reinterpret_cast<int*>(smem_raw + RING_BYTES + NW * EPI_BYTES);
+  // [ring][epilogue scratch: NW x EPI_BYTES, not with PP][expert table: E x (tiles inclusive, row end)]
+  int* etab = reinterpret_cast<int*>(smem_raw + RING_BYTES + (PP ? 0 : NW * EPI_BYTES));
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -943,8 +947,12 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
 
   // ---- epilogue of one tile: acc -> (SwiGLU) -> LDS scratch -> 16-byte row-contiguous stores -----------
   T* __restrict__ out = static_cast<T*>(a.out);
-  unsigned char* scratch = smem_raw + RING_BYTES + wave * EPI_BYTES;
+  static_assert(!PP || NW * EPI_BYTES <= STAGE_BYTES, "epilogue scratch must fit the free ring stage");
   auto epilogue = [&](const TileCoord& tc) {
+    // PP: the ring stage consumed last is free until the next tile's first memory phase refills it (the
+    // tile loop puts a barrier between this epilogue and that refill)
+    unsigned char* scratch = PP ? smem_raw + ((g + NSTAGE - 1) & (NSTAGE - 1)) * STAGE_BYTES + wave * EPI_BYTES
+                                : smem_raw + RING_BYTES + wave * EPI_BYTES;
     // scratch row r keeps its EPI_CPR 16-byte chunks at slots chunk ^ swz(r): the 8-byte writes of a
     // wave and the 16-byte read-back both spread over all banks
     auto swz = [](int r) { return EPI_CPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3); };
@@ -1061,6 +1069,12 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     int raw2[NXLD];
     load_rows(c2, raw2);
     epilogue(c0);
+    if (PP) {
+      // every wave is done with its scratch before any wave's DMA of the next tile lands in that stage
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+    }
     if (t1 < 0) {
       // The compiler folds this exit into the loop's back edge and then assumes, inside the slice loop, that
       // the row-index loads above may still be in flight (nobody consumes them on this path): it would drain
@@ -1154,7 +1168,7 @@ template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool PP
 static int launch_persistent(GemmArgs a, hipStream_t s) {
   constexpr int BN = GLU ? BNW / 2 : BNW;
   constexpr int NW = WM * WN;
-  const size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T) + (size_t)NW * (NW > 4 ? 2048 : 4096) + (size_t)a.E * 8;
+  const size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T) + (PP ? 0 : (size_t)NW * (NW > 4 ? 2048 : 4096)) + (size_t)a.E * 8;
   auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, BK, PP>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
