@@ -34,8 +34,8 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # for FETCH_SIZE, x1.000 for WRITE_SIZE); the summaries are under profiles/.  A counter cannot be read
 # from inside this process, so the figures are recorded here and are null for other workloads.
 MEASURED_TRAFFIC_BYTES = {
-    "granite-3b-a800m": 1464.2e6 + 268.6e6,   # up-projection GEMM: fetch + write
-    "decode-fp8": 758.0e6 + 1.1e6,            # fp8 up-projection: fetch + write
+    "granite-3b-a800m": 1555.8e6 + 268.4e6,   # up-projection GEMM: fetch + write
+    "decode-fp8": 757.6e6 + 1.1e6,            # fp8 up-projection: fetch + write
 }
 
 
