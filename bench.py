@@ -122,11 +122,24 @@ def cpu_baseline(w, inputs, sample_tokens, iters=3):
         run()
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
-    return {
+    out = {
         "value": sample_tokens / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
         "sample": f"first {sample_tokens} tokens of the workload, fp32 eager per-expert loop, 1 warm-up + {iters} "
                   f"timed forwards, median {med * 1e3:.1f} ms; host has {os.cpu_count()} logical cpus",
     }
+    if not w.fp8 and w.dtype == torch.bfloat16:
+        # the same loop in the model dtype (host bf16 GEMMs are often slower than fp32): one warm-up, one timed
+        xb, gb, fb, pb = x.bfloat16(), gate_w.bfloat16(), w_fc.bfloat16(), w_proj.bfloat16()
+
+        def run_bf16():
+            _, gates, idx = oracle.route(xb, gb, w.k, bias=bias)
+            return oracle.experts_eager(xb, gates, idx, fb, pb)
+
+        run_bf16()
+        t0 = time.perf_counter()
+        run_bf16()
+        out["value_model_dtype"] = sample_tokens / (time.perf_counter() - t0)
+    return out
 
 
 def main():

@@ -87,7 +87,7 @@ class ParameterizedExperts(nn.Module):
                 num_tokens_per_expert: torch.Tensor | None = None,
                 sorted_expert_idxs: torch.Tensor | None = None, sorted_scattered_idxs: torch.Tensor | None = None,
                 expert_offsets: torch.Tensor | None = None, gates: torch.Tensor | None = None,
-                grouped_in: bool = False, grouped_out: bool = False) -> torch.Tensor:
+                grouped_in: bool = False, grouped_out: bool = False, combine_tail: tuple | None = None) -> torch.Tensor:
         if is_kernel_allowed(Kernel.scattermoe):
             assert self.bias is None
             if self.weight_q is not None:
@@ -102,6 +102,7 @@ class ParameterizedExperts(nn.Module):
                 gates=gates,
                 grouped_in=grouped_in,
                 grouped_out=grouped_out,
+                combine_tail=combine_tail,
             )
         weight = self.dense_weight()
         pieces = input.split(num_tokens_per_expert.tolist(), dim=0)
@@ -199,25 +200,49 @@ class MoE(nn.Module):
 
     # ---------------------------------------------------------------------------------------------
 
-    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+    def forward(self, hidden_states: torch.Tensor, residual: torch.Tensor | None = None,
+                residual_scale: float | None = None) -> torch.Tensor:
+        """moe.py:212-244.  ``residual`` / ``residual_scale`` are an extension: with them the result is
+        ``moe(hidden_states) * residual_scale + residual``, i.e. the two lines the transformer block runs after
+        its mlp_block (mixins/dense/layer.py:61-66); on the kernel branch they -- and the shared-expert sum --
+        are folded into the combine pass, with the roundings of the separate operations."""
         if not self.use_padding_free_transformer:
             batch_size, sequence_length, _ = hidden_states.shape
 
         hidden_states = hidden_states.view(-1, self.hidden_size)
+        if residual is not None:
+            residual = residual.reshape(-1, self.hidden_size)
 
         router_logits, router_weights, selected_experts = self._compute_routing_weights(hidden_states)
-        moe_output = self._compute_experts(hidden_states, router_weights, selected_experts)
 
-        if self.shared_intermediate_size is None:
-            hidden_states = moe_output
+        # the tail can only be folded in where nothing sits between the expert sum and it
+        fuse_tail = (
+            is_kernel_allowed(Kernel.scattermoe)
+            and isinstance(self.dropout, nn.Identity)
+            and (self.shared_intermediate_size is not None or residual is not None or residual_scale is not None)
+        )
+        if fuse_tail:
+            shared = None if self.shared_intermediate_size is None else self._compute_shared_experts(hidden_states)
+            hidden_states = self._compute_experts(hidden_states, router_weights, selected_experts,
+                                                  tail=(shared, residual, residual_scale))
         else:
-            hidden_states = moe_output + self._compute_shared_experts(hidden_states)
-        del moe_output
+            moe_output = self._compute_experts(hidden_states, router_weights, selected_experts)
+            if self.shared_intermediate_size is None:
+                hidden_states = moe_output
+            else:
+                hidden_states = moe_output + self._compute_shared_experts(hidden_states)
+            del moe_output
 
         if not self.use_padding_free_transformer:
             hidden_states = hidden_states.reshape(batch_size, sequence_length, self.hidden_size)
 
         hidden_states = self.dropout(hidden_states)
+
+        if not fuse_tail:
+            if residual_scale is not None:
+                hidden_states = hidden_states * residual_scale
+            if residual is not None:
+                hidden_states = hidden_states + residual.reshape(hidden_states.shape)
 
         aux_loss = (
             self._compute_switch_loss(
@@ -261,8 +286,10 @@ class MoE(nn.Module):
         return router_logits, router_weights, selected_experts
 
     def _compute_experts(self, hidden_states: torch.Tensor, router_weights: torch.Tensor,
-                         selected_experts: torch.Tensor) -> torch.Tensor:
+                         selected_experts: torch.Tensor, tail: tuple | None = None) -> torch.Tensor:
+        """``tail`` = (shared-expert output, residual, residual_scale) to fold into the combine (kernel branch)."""
         if is_kernel_allowed(Kernel.scattermoe):
+            shared, residual, residual_scale = tail if tail is not None else (None, None, None)
             sorted_expert_idxs, sorted_scattered_idxs, expert_offsets = ops.sort_bin(selected_experts, self.num_experts)
 
             if self.c_fc.weight_q is not None:
@@ -272,7 +299,7 @@ class MoE(nn.Module):
                                                   self.top_k, sorted_scattered_idxs, expert_offsets)
                 hidden_states = ops.down_fp8(hidden_states, self.c_proj.weight_q, self.c_proj.weight_scale,
                                              sorted_scattered_idxs, expert_offsets)
-                hidden_states = ops.combine(hidden_states, router_weights)
+                hidden_states = ops.combine(hidden_states, router_weights, shared, residual, residual_scale)
             else:
                 if self._fused_swiglu:
                     assert self.c_fc.bias is None
@@ -296,6 +323,7 @@ class MoE(nn.Module):
                     expert_offsets=expert_offsets,
                     grouped_in=True,
                     gates=router_weights,
+                    combine_tail=tail,
                 )
             hidden_states = self.dropout(hidden_states)
         else:
@@ -317,6 +345,18 @@ class MoE(nn.Module):
         return hidden_states
 
     def _compute_shared_experts(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        """moe.py:311-315.  On the kernel branch the dense SwiGLU MLP runs as a one-expert grouped GEMM (SwiGLU
+        in the up-projection's epilogue)."""
+        if (
+            is_kernel_allowed(Kernel.scattermoe) and self._fused_swiglu and hidden_states.is_cuda
+            and self.c_fc_shared.bias is None and self.c_proj_shared.bias is None
+            and hidden_states.dtype in (torch.bfloat16, torch.float16) and not torch.is_grad_enabled()
+        ):
+            T = hidden_states.shape[0]
+            rows = torch.arange(T, dtype=torch.int32, device=hidden_states.device)
+            offsets = torch.full((1,), T, dtype=torch.int32, device=hidden_states.device)
+            act = ops.up_swiglu(hidden_states, self.c_fc_shared.weight.unsqueeze(0), 1, rows, offsets)
+            return ops.scattered_gemm(act, self.c_proj_shared.weight.unsqueeze(0), 1, rows, offsets, True, True)
         hidden_states = self.c_fc_shared(hidden_states)
         hidden_states = self.act(hidden_states)
         hidden_states = self.c_proj_shared(hidden_states)

@@ -213,9 +213,14 @@ def scattered_gemm(inputs: torch.Tensor, weight: torch.Tensor, k: int, sorted_sc
     return out
 
 
-def combine(o: torch.Tensor, gates: torch.Tensor) -> torch.Tensor:
-    """y[t] = sum_j gates[t, j] * o[t*k + j]  with o (T*k, H), gates (T, k)."""
-    _dev(o, gates)
+def combine(o: torch.Tensor, gates: torch.Tensor, shared: torch.Tensor | None = None,
+            residual: torch.Tensor | None = None, residual_scale: float | None = None) -> torch.Tensor:
+    """y[t] = sum_j gates[t, j] * o[t*k + j]  with o (T*k, H), gates (T, k).
+
+    Optionally folds the tail of the transformer block into the same pass, each step rounded to the
+    dtype like the separate torch operations: ``+ shared`` (shared-expert output, moe.py:214),
+    ``* residual_scale`` (m_residual) and ``+ residual`` (mixins/dense/layer.py:61-66)."""
+    _dev(o, gates, shared, residual)
     _no_grad(o, gates)
     o = o.contiguous()
     gates = gates.contiguous()
@@ -223,29 +228,43 @@ def combine(o: torch.Tensor, gates: torch.Tensor) -> torch.Tensor:
     H = o.shape[1]
     if o.shape[0] != T * k or gates.dtype != o.dtype:
         raise ValueError("o must be (T*k, H) and gates (T, k) of the same dtype")
+    for name, t in (("shared", shared), ("residual", residual)):
+        if t is not None and (tuple(t.shape) != (T, H) or t.dtype != o.dtype):
+            raise ValueError(f"{name} must be (T, H) in the dtype of o")
     y = torch.empty((T, H), dtype=o.dtype, device=o.device)
     with _stage("combine"):
-        check(_lib.load().mi_moe_combine(_ptr(o), _ptr(gates), _ptr(y), T, k, H, _code(o.dtype), _stream()))
+        if shared is None and residual is None and residual_scale is None:
+            check(_lib.load().mi_moe_combine(_ptr(o), _ptr(gates), _ptr(y), T, k, H, _code(o.dtype), _stream()))
+        else:
+            shared = None if shared is None else shared.contiguous()
+            residual = None if residual is None else residual.contiguous()
+            check(_lib.load().mi_moe_combine_block_tail(
+                _ptr(o), _ptr(gates), _ptr(shared), _ptr(residual),
+                1.0 if residual_scale is None else float(residual_scale), int(residual_scale is not None),
+                _ptr(y), T, k, H, _code(o.dtype), _stream()))
     return y
 
 
 def scattered_experts(inputs: torch.Tensor, expert_weights: torch.Tensor, k: int,
                       sorted_expert_idxs: torch.Tensor, sorted_scattered_idxs: torch.Tensor,
                       expert_offsets: torch.Tensor, gates: torch.Tensor | None = None, grouped_in: bool = False,
-                      grouped_out: bool = False) -> torch.Tensor:
+                      grouped_out: bool = False, combine_tail: tuple | None = None) -> torch.Tensor:
     """Drop-in for the external ``scattered_experts`` (moe.py:91-101).
 
     ``expert_weights`` is the (E, in, out) view the reference passes (``weight.permute(0, 2, 1)``);
     ``sorted_expert_idxs`` is accepted for signature compatibility (the kernels derive the expert of
     a row from ``expert_offsets``).  With ``gates`` (T, k_g) the (L, out) result is contracted to
-    (T, out)."""
+    (T, out); ``combine_tail`` = (shared, residual, residual_scale) is an extension handed on to
+    :func:`combine`."""
     del sorted_expert_idxs
     w = _native_weight(expert_weights)
     if gates is not None and grouped_out:
         raise ValueError("gates need the output in flat-slot order (grouped_out=False)")
     out = scattered_gemm(inputs, w, k, sorted_scattered_idxs, expert_offsets, grouped_in, grouped_out)
+    if combine_tail is not None and gates is None:
+        raise ValueError("combine_tail needs gates")
     if gates is not None:
-        out = combine(out, gates.to(out.dtype))
+        out = combine(out, gates.to(out.dtype), *(combine_tail or ()))
     return out
 
 

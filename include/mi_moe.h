@@ -150,6 +150,20 @@ int mi_moe_combine(const void* o, const void* gates, void* y, int T, int k, int 
                    mi_moe_stream_t stream);
 
 /*
+ * Combine with the tail of the transformer block folded in:
+ *     r = round(sum_j gates[t, j] * o[t*k + j, :])          (the call above)
+ *     r = round(r + shared[t, :])        if shared          (shared experts, moe.py:214)
+ *     r = round(r * residual_scale)      if has_scale       (m_residual, mixins/dense/layer.py:61-62)
+ *     y[t, :] = round(r + residual[t, :]) if residual       (mixins/dense/layer.py:64)
+ * Every step is rounded to `dtype` as the separate torch operations round it, so the result equals
+ * running them after mi_moe_combine bit for bit; two (T, H) round trips through HBM less.
+ *   shared, residual (T, H) of `dtype` or NULL.
+ */
+int mi_moe_combine_block_tail(const void* o, const void* gates, const void* shared, const void* residual,
+                              float residual_scale, int has_scale, void* y, int T, int k, int H, int dtype,
+                              mi_moe_stream_t stream);
+
+/*
  * Decode-shape variants with fp8 (OCP e4m3fn) expert weights and one fp32 scale per output channel.
  * No counterpart in the reference (its fp8 support wraps nn.Linear only, lm_engine/fp8.py:63-73);
  * semantics = dequantise (w * scale[:, None]) then the two calls above.

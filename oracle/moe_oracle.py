@@ -232,8 +232,11 @@ def moe_forward(x: torch.Tensor, gate_weight: torch.Tensor, w_fc: torch.Tensor, 
                 bias: torch.Tensor | None = None, logits: torch.Tensor | None = None,
                 w_fc_scale: torch.Tensor | None = None, w_proj_scale: torch.Tensor | None = None,
                 compute_dtype: torch.dtype | None = torch.float32,
-                shared_fc: torch.Tensor | None = None, shared_proj: torch.Tensor | None = None) -> OracleOutput:
-    """moe.py:212-244 in eval mode with the eager expert branch; x is (T, H)."""
+                shared_fc: torch.Tensor | None = None, shared_proj: torch.Tensor | None = None,
+                residual: torch.Tensor | None = None, residual_scale: float | None = None) -> OracleOutput:
+    """moe.py:212-244 in eval mode with the eager expert branch; x is (T, H).  With ``residual`` /
+    ``residual_scale`` also the two lines the transformer block runs after the layer
+    (mixins/dense/layer.py:61-66): y * m_residual + residual."""
     E = w_fc.shape[0]
     logits, gates, experts = route(x, gate_weight, k, bias=bias, logits=logits)
     if w_fc_scale is not None:
@@ -246,6 +249,10 @@ def moe_forward(x: torch.Tensor, gate_weight: torch.Tensor, w_fc: torch.Tensor, 
         sf = shared_fc if compute_dtype is None else shared_fc.to(compute_dtype)
         sp = shared_proj if compute_dtype is None else shared_proj.to(compute_dtype)
         y = y + F.linear(swiglu(F.linear(xs, sf)), sp)
+    if residual_scale is not None:  # mixins/dense/layer.py:61-62
+        y = y * residual_scale
+    if residual is not None:        # mixins/dense/layer.py:64
+        y = y + (residual if compute_dtype is None else residual.to(compute_dtype))
     se, ss, off = sort_bin(experts, E)
     return OracleOutput(y, logits, gates, experts, se, ss, off)
 

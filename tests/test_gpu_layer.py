@@ -134,6 +134,67 @@ def test_layer_shared_experts(device):
     torch.testing.assert_close(y.cpu().float(), ref.y, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shared_size", [None, 96])
+def test_layer_block_tail(device, dtype, shared_size):
+    """Shared experts, m_residual and the residual folded into the combine pass: bit-identical to the same
+    module followed by the separate torch operations, and within tolerance of the fp32 oracle."""
+    from dolomite_engine_amd import Kernel, MoE, enable_kernels
+
+    torch.manual_seed(11)
+    m = MoE(hidden_size=128, intermediate_size=64, shared_intermediate_size=shared_size, num_experts=8,
+            num_experts_per_tok=2, activation_function="swiglu", add_bias=False, dropout=0.0, init_method="normal",
+            initializer_range=0.05, m_width=None, num_layers=1, use_padding_free_transformer=True)
+    m = m.to(dtype).to(device).eval()
+    x = torch.randn(333, 128, device=device, dtype=dtype)
+    res = torch.randn(333, 128, device=device, dtype=dtype)
+    scale = 0.22
+    with torch.no_grad(), enable_kernels([Kernel.scattermoe]):
+        fused = m(x, residual=res, residual_scale=scale)
+        plain = m(x)                      # shared experts (if any) are folded in here too
+        unfused = plain * scale + res     # the block's own two operations
+        only_scale = m(x, residual_scale=scale)
+        only_res = m(x, residual=res)
+    assert torch.equal(fused, unfused)
+    assert torch.equal(only_scale, plain * scale)
+    assert torch.equal(only_res, plain + res)
+    kw = {} if shared_size is None else dict(shared_fc=m.c_fc_shared.weight.cpu(), shared_proj=m.c_proj_shared.weight.cpu())
+    ref = oracle.moe_forward(x.cpu(), m.gate.weight.cpu(), m.c_fc.weight.cpu(), m.c_proj.weight.cpu(), 2,
+                             residual=res.cpu(), residual_scale=scale, **kw)
+    torch.testing.assert_close(fused.cpu().float(), ref.y, rtol=2e-2, atol=2e-2)
+    # the eager branch takes the same arguments
+    with torch.no_grad():
+        eager = m(x, residual=res, residual_scale=scale)
+    torch.testing.assert_close(eager.float(), fused.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_combine_block_tail_matches_separate_ops(device):
+    """mi_moe_combine_block_tail == mi_moe_combine followed by torch's add / mul / add, bit for bit, for
+    every subset of the three optional steps (vector and scalar kernels)."""
+    from dolomite_engine_amd import ops
+
+    g = torch.Generator().manual_seed(5)
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        for T, k, H in ((70, 8, 1536), (33, 3, 100)):
+            o = torch.randn(T * k, H, generator=g).to(dtype).to(device)
+            gates = torch.softmax(torch.randn(T, k, generator=g), -1).to(dtype).to(device)
+            shared = torch.randn(T, H, generator=g).to(dtype).to(device)
+            res = torch.randn(T, H, generator=g).to(dtype).to(device)
+            base = ops.combine(o, gates)
+            for use_sh in (False, True):
+                for scale in (None, 0.3):
+                    for use_res in (False, True):
+                        got = ops.combine(o, gates, shared if use_sh else None, res if use_res else None, scale)
+                        want = base
+                        if use_sh:
+                            want = want + shared
+                        if scale is not None:
+                            want = want * scale
+                        if use_res:
+                            want = want + res
+                        assert torch.equal(got, want), (dtype, T, k, H, use_sh, scale, use_res)
+
+
 def test_kernel_branch_refuses_grad(device):
     from dolomite_engine_amd import Kernel, MoE, enable_kernels
 
