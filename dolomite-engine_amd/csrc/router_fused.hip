@@ -26,14 +26,50 @@ template <> struct RMfma<f16_t> {
   }
 };
 
-__device__ __forceinline__ uint32_t router_ordered_key(float v) {
-  uint32_t u = __float_as_uint(v);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;
-  if (u == 0x80000000u) u = 0u;
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+#define ROUTER_KMAX 8
+
+// The logits are values of a 16-bit type, so (value, expert) orders as ONE 32-bit integer:
+//   bits 31..16  the value's bit pattern made monotonic (NaN largest, -0 == +0),
+//   bits 15..0   0xffff - expert (the lower expert wins a tie).
+// The value is recovered from the winner's key, so no second array follows the keys around.
+template <typename T> struct Bits16;
+template <> struct Bits16<bf16_t> {
+  static constexpr uint32_t INF = 0x7f80u;
+  static __device__ __forceinline__ uint32_t of(float rounded) { return __float_as_uint(rounded) >> 16; }
+  static __device__ __forceinline__ float value(uint32_t u) { return __uint_as_float(u << 16); }
+};
+template <> struct Bits16<f16_t> {
+  static constexpr uint32_t INF = 0x7c00u;
+  static __device__ __forceinline__ uint32_t of(float rounded) {
+    const f16_t h = (f16_t)rounded;
+    return (uint32_t)__builtin_bit_cast(uint16_t, h);
+  }
+  static __device__ __forceinline__ float value(uint32_t u) {
+    const uint16_t b = (uint16_t)u;
+    return (float)__builtin_bit_cast(f16_t, b);
+  }
+};
+template <typename T>
+__device__ __forceinline__ uint32_t router_ordered16(uint32_t u) {
+  if ((u & 0x7fffu) > Bits16<T>::INF) return 0xffffu;  // NaN
+  if (u == 0x8000u) u = 0u;                             // -0 == +0
+  return (u & 0x8000u) ? (~u & 0xffffu) : (u | 0x8000u);
+}
+template <typename T>
+__device__ __forceinline__ float router_value_of_key(uint32_t key) {
+  const uint32_t o = key >> 16;
+  return Bits16<T>::value((o & 0x8000u) ? (o ^ 0x8000u) : (~o & 0xffffu));
 }
 
-#define ROUTER_KMAX 8
+// max over the four lanes (q = 0..3) that hold one token's candidates: lanes l, l^16, l^32, l^48.
+// v_permlane16_swap with both operands x leaves {x of the even row, x of the odd row} of each row pair in the
+// two results, v_permlane32_swap the same for the two halves; a max of the two results is the butterfly step.
+__device__ __forceinline__ uint32_t router_max4(uint32_t x) {
+  const auto a = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+  const uint32_t m = a[0] > a[1] ? a[0] : a[1];
+  const auto b = __builtin_amdgcn_permlane32_swap(m, m, false, false);
+  return b[0] > b[1] ? b[0] : b[1];
+}
 
 // Epilogue for one group of 16 tokens: lane (r = token, q) holds acc[eb][i] = logit of expert
 // 16*eb + 4*q + i.  Rounds to the model dtype, adds the optional bias, optionally stores the logits,
@@ -43,8 +79,7 @@ __device__ __forceinline__ void router_epilogue(const f32x4 (&acc)[4], int t, bo
                                                 const float* __restrict__ bias, int E, int k,
                                                 T* __restrict__ logits_out, T* __restrict__ gates,
                                                 int32_t* __restrict__ idx) {
-  uint64_t keys[16];
-  float vals[16];
+  uint32_t keys[16];
 #pragma unroll
   for (int eb = 0; eb < 4; ++eb) {
 #pragma unroll
@@ -52,8 +87,7 @@ __device__ __forceinline__ void router_epilogue(const f32x4 (&acc)[4], int t, bo
       const int e = eb * 16 + 4 * q + i;
       float v = Elt<T>::round(acc[eb][i]);
       if (bias != nullptr && e < E) v = Elt<T>::round(v + bias[e]);
-      vals[eb * 4 + i] = v;
-      keys[eb * 4 + i] = e < E ? (((uint64_t)router_ordered_key(v) << 32) | (uint32_t)(~(uint32_t)e)) : 0ull;
+      keys[eb * 4 + i] = e < E ? ((router_ordered16<T>(Bits16<T>::of(v)) << 16) | (0xffffu - (uint32_t)e)) : 0u;
       if (logits_out != nullptr && tvalid && e < E) Elt<T>::store(logits_out + (size_t)t * E + e, v);
     }
   }
@@ -64,31 +98,15 @@ __device__ __forceinline__ void router_epilogue(const f32x4 (&acc)[4], int t, bo
     wv[j] = 0.f;
     wi[j] = 0;
     if (j < k) {
-      uint64_t best = 0ull;
-      float bv = 0.f;
+      uint32_t best = keys[0];
 #pragma unroll
-      for (int c = 0; c < 16; ++c) {
-        if (keys[c] > best) {
-          best = keys[c];
-          bv = vals[c];
-        }
-      }
-#pragma unroll
-      for (int off = 16; off <= 32; off <<= 1) {
-        uint32_t lo = __shfl_xor((uint32_t)best, off, MI_WAVE);
-        uint32_t hi = __shfl_xor((uint32_t)(best >> 32), off, MI_WAVE);
-        float ov = __shfl_xor(bv, off, MI_WAVE);
-        uint64_t o = ((uint64_t)hi << 32) | lo;
-        if (o > best) {
-          best = o;
-          bv = ov;
-        }
-      }
+      for (int c = 1; c < 16; ++c) best = keys[c] > best ? keys[c] : best;
+      best = router_max4(best);
 #pragma unroll
       for (int c = 0; c < 16; ++c)
-        if (keys[c] == best) keys[c] = 0ull;
-      wv[j] = bv;
-      wi[j] = (int)(~(uint32_t)best);
+        if (keys[c] == best) keys[c] = 0u;
+      wv[j] = router_value_of_key<T>(best);
+      wi[j] = (int)(0xffffu - (best & 0xffffu));
     }
   }
   if (q == 0 && tvalid) {
@@ -180,6 +198,118 @@ __global__ __launch_bounds__(256) void router_fused_kernel(const T* __restrict__
 #pragma unroll
     for (int eb = 0; eb < 4; ++eb) a4[eb] = acc[eb][g];
     router_epilogue<T>(a4, t, t < Trows, q, bias, E, k, logits_out, gates, idx);
+  }
+}
+
+// Many tokens, gate weights held in LDS.  The kernel above re-reads the gate weights (E x H) from L2 for every
+// 32 tokens -- more bytes than x itself -- and runs four waves per CU.  Here a workgroup of eight waves copies the
+// weights into LDS once (row pitch 2H + 16 bytes: the 16 rows of a fragment read then start in 16 different
+// 16-byte bank groups) and then walks 16-token groups, one per wave and turn; x streams through a register ring
+// DEPTH K steps deep (3 with eight waves: about 48 KB in flight per CU), and only the ceil(E / 16) expert blocks that exist are
+// multiplied.
+// With fewer than eight groups per CU the launch uses fewer waves per workgroup (so that every CU takes part)
+// and a deeper ring per wave (DEPTH 6) to keep as many bytes in flight.
+#define ROUTER_LDS_WAVES 8
+template <typename T, int DEPTH>
+__global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel(
+    const T* __restrict__ x, const T* __restrict__ gw, const float* __restrict__ bias, int Trows, int H, int E, int k,
+    T* __restrict__ logits_out, T* __restrict__ gates, int32_t* __restrict__ idx) {
+  typedef typename RMfma<T>::vec frag_t;
+  extern __shared__ __attribute__((aligned(16))) unsigned char wlds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int pitch = H * (int)sizeof(T) + 16;
+  // ---- gate weights -> LDS (16-byte pieces; H % 16 == 0 is checked on the host) ----
+  const int nwaves = blockDim.x >> 6;
+  const int nsteps = (H + 63) >> 6;
+  const int ngroups = (Trows + 15) >> 4;
+  const int stride = gridDim.x * nwaves;
+  int grp = blockIdx.x * nwaves + wave;
+
+  // x ring of the wave's current group; the first DEPTH steps of a group are requested before the previous
+  // group's epilogue (for the first group: before the weights are copied), so their latency is hidden
+  const T* xrow = x;
+  u32x4 xr[DEPTH][2];
+  auto load_x = [&](int step, u32x4 (&dst)[2]) {
+    const int kpos = step * 64 + q * 16;
+    dst[0] = dst[1] = (u32x4){0u, 0u, 0u, 0u};
+    if (step < nsteps && kpos < H) {  // the MFMA runs on all lanes: out-of-range k contributes zeros
+      dst[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xrow + kpos));
+      dst[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xrow + kpos + 8));
+    }
+  };
+  auto open_group = [&](int g) {
+    int t = g * 16 + r;
+    if (t > Trows - 1) t = Trows - 1;
+    xrow = x + (size_t)t * H;
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) load_x(d, xr[d]);
+  };
+  if (grp < ngroups) open_group(grp);
+
+  // ---- gate weights -> LDS (16-byte pieces; H % 16 == 0 is checked on the host) ----
+  // eight loads in flight per thread: one load-wait-store per iteration would pay an L2 latency per piece
+  const int pieces_per_row = H * (int)sizeof(T) / 16;
+  const int pieces = E * pieces_per_row;
+  for (int p0 = threadIdx.x; p0 < pieces; p0 += 8 * blockDim.x) {
+    u32x4 v[8];
+    int dst[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int p = p0 + i * blockDim.x;
+      dst[i] = -1;
+      if (p < pieces) {
+        const int e = p / pieces_per_row, c = p - e * pieces_per_row;
+        dst[i] = e * pitch + c * 16;
+        v[i] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned char*>(gw) + (size_t)p * 16);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (dst[i] >= 0) *reinterpret_cast<u32x4*>(wlds + dst[i]) = v[i];
+  }
+  __syncthreads();
+
+  const int neb = (E + 15) >> 4;
+  int wbase[4];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) {
+    int e = eb * 16 + r;
+    if (e > E - 1) e = E - 1;
+    wbase[eb] = e * pitch;
+  }
+  while (grp < ngroups) {
+    f32x4 acc[4];
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) acc[eb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < nsteps; s0 += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int step = s0 + d;
+        if (step < nsteps) {
+          const int kbyte = (step * 64 + q * 16) * (int)sizeof(T);
+          const bool valid = step * 64 + q * 16 < H;
+          const u32x4 x0 = xr[d][0], x1 = xr[d][1];
+          load_x(step + DEPTH, xr[d]);
+#pragma unroll
+          for (int eb = 0; eb < 4; ++eb) {
+            if (eb < neb) {
+              u32x4 w0 = {0u, 0u, 0u, 0u}, w1 = {0u, 0u, 0u, 0u};
+              if (valid) {
+                w0 = *reinterpret_cast<const u32x4*>(wlds + wbase[eb] + kbyte);
+                w1 = *reinterpret_cast<const u32x4*>(wlds + wbase[eb] + kbyte + 16);
+              }
+              acc[eb] = RMfma<T>::run(__builtin_bit_cast(frag_t, w0), __builtin_bit_cast(frag_t, x0), acc[eb]);
+              acc[eb] = RMfma<T>::run(__builtin_bit_cast(frag_t, w1), __builtin_bit_cast(frag_t, x1), acc[eb]);
+            }
+          }
+        }
+      }
+    }
+    const int t = grp * 16 + r;
+    grp += stride;
+    if (grp < ngroups) open_group(grp);
+    router_epilogue<T>(acc, t, t < Trows, q, bias, E, k, logits_out, gates, idx);
   }
 }
 
@@ -381,6 +511,25 @@ static int launch_router(const void* x, const void* gw, const float* bias, int T
     hipLaunchKernelGGL((router_fused_small_kernel<T>), dim3(mi_ceil_div(T_, 16)), dim3(1024), 0, s,
                        static_cast<const T*>(x), static_cast<const T*>(gw), bias, T_, H, E, k,
                        static_cast<T*>(logits_out), static_cast<T*>(gates), idx);
+    return mi_launch_status();
+  }
+  // gate weights fit in LDS next to nothing else: the LDS-resident kernel
+  const size_t wbytes = (size_t)E * ((size_t)H * sizeof(T) + 16);
+  if (wbytes <= 156u * 1024u) {
+    int dev = 0, cus = 0;
+    hipError_t e;
+    if ((e = hipGetDevice(&dev)) != hipSuccess) return (int)e;
+    if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return (int)e;
+    const int groups = mi_ceil_div(T_, 16);
+    const int blocks = groups < cus ? groups : cus;
+    int waves = mi_ceil_div(groups, blocks);
+    if (waves > ROUTER_LDS_WAVES) waves = ROUTER_LDS_WAVES;
+    auto kern = waves > 4 ? router_fused_lds_kernel<T, 3> : router_fused_lds_kernel<T, 6>;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)wbytes);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(waves * 64), wbytes, s, static_cast<const T*>(x),
+                       static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out),
+                       static_cast<T*>(gates), idx);
     return mi_launch_status();
   }
   constexpr int TG = 2;
