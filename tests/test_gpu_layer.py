@@ -208,7 +208,7 @@ def test_kernel_branch_refuses_grad(device):
             m(x)
 
 
-@pytest.mark.parametrize("name", ["granite-1b-a400m", "granite-3b-a800m"])
+@pytest.mark.parametrize("name", ["granite-1b-a400m", "granite-3b-a800m", "mixtral"])
 def test_full_size_properties(device, name):
     """Full benchmark sizes: size-independent properties instead of a CPU recomputation.
 
@@ -241,7 +241,7 @@ def test_full_size_properties(device, name):
     assert torch.equal(y2.float(), 2 * y.float())
     # sampled tokens against the oracle (same logits -> same routing)
     g = torch.Generator().manual_seed(0)
-    sample = torch.randperm(w.T, generator=g)[:256]
+    sample = torch.randperm(w.T, generator=g)[:256 if w.I <= 4096 else 48]  # the oracle runs on the host
     ref = oracle.moe_forward(inputs["x"][sample], inputs["gate_w"], inputs["w_fc"], inputs["w_proj"], w.k,
                              bias=inputs["bias"], logits=logits.cpu()[sample])
     assert torch.equal(idx_c[sample], ref.experts)
