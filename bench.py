@@ -65,7 +65,7 @@ class StageTimer:
         return {n: sum(a.elapsed_time(b) for a, b in evs) / len(evs) for n, evs in self.events.items()}
 
 
-def build_module(w, inputs, device):
+def build_module(w, inputs, device, fp8_tiled=True):
     import torch
 
     from dolomite_engine_amd import MoE
@@ -79,13 +79,10 @@ def build_module(w, inputs, device):
     with torch.no_grad():
         m.gate.weight.copy_(inputs["gate_w"])
         if w.fp8:
-            m.c_fc.weight = None
-            m.c_proj.weight = None
-            m.c_fc.weight_q = inputs["w_fc"].to(device)
-            m.c_fc.weight_scale = inputs["fc_scale"].to(device)
-            m.c_proj.weight_q = inputs["w_proj"].to(device)
-            m.c_proj.weight_scale = inputs["proj_scale"].to(device)
-            m.c_fc.weight_scale_dtype = m.c_proj.weight_scale_dtype = w.dtype
+            m.c_fc.set_fp8_weight(inputs["w_fc"].to(device), inputs["fc_scale"].to(device), w.dtype,
+                                  tiled=fp8_tiled, glu=True)
+            m.c_proj.set_fp8_weight(inputs["w_proj"].to(device), inputs["proj_scale"].to(device), w.dtype,
+                                    tiled=fp8_tiled, glu=False)
         else:
             m.c_fc.weight.copy_(inputs["w_fc"])
             m.c_proj.weight.copy_(inputs["w_proj"])
@@ -150,6 +147,8 @@ def main():
     ap.add_argument("--workload", default="granite-3b-a800m")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=None)
+    ap.add_argument("--fp8-row-major", action="store_true",
+                    help="decode workload: keep the fp8 expert weights row-major instead of in the streamed-tile layout")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy so that a rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE run of this command contains a kernel of known traffic to scale by")
@@ -173,7 +172,7 @@ def main():
 
     w = oracle.WORKLOADS[args.workload]
     inputs = oracle.make_inputs(w)
-    m = build_module(w, inputs, device)
+    m = build_module(w, inputs, device, fp8_tiled=not args.fp8_row_major)
     x = inputs["x"].to(device)
     T, H, E, k, I = w.T, w.H, w.E, w.k, w.I
     L = T * k
@@ -238,7 +237,8 @@ def main():
         "dtype": "bf16" if not w.fp8 else "bf16 activations, fp8-e4m3 weights", "data": "synthetic",
         "config": {"workload": w.name, "tokens": T, "hidden": H, "experts": E, "top_k": k, "intermediate": I,
                    "expert_load": "zipf(1.1) first-choice" if w.zipf_s else "near-uniform",
-                   "experts_touched": touched, "max_over_min_load": float(counts.max()) / max(1.0, float(counts.min()))},
+                   "experts_touched": touched, "max_over_min_load": float(counts.max()) / max(1.0, float(counts.min())),
+                   **({"fp8_weight_layout": "row-major" if args.fp8_row_major else "streamed tiles"} if w.fp8 else {})},
         "layer_tflops": flops / (elapsed / args.steps) / 1e12,
         "stages_ms": stages,
         "roofline": roofline,

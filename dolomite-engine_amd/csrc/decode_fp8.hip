@@ -63,7 +63,8 @@ struct DecodeArgs {
   const int32_t* expert_offsets;
   int L, K, N, E, kdiv;
   int gather, scatter;
-  int groups_per_expert;  // workgroups per expert
+  int groups_per_expert;  // workgroups per expert (streaming kernel: wave units per expert)
+  int tiled;              // weights are in the streamed-tile layout (streaming kernel only)
 };
 
 template <typename T, bool GLU, int KSPLIT>
@@ -199,7 +200,12 @@ __device__ __forceinline__ constexpr int dec_waitcnt(int vm, int lgkm) {
 
 template <int V> struct dec_int { static constexpr int value = V; };
 
-template <typename T, bool GLU>
+// TILED: the weights are stored as the kernel streams them -- [expert][wave unit][K stage][4 KB], each 4 KB block
+// being the LDS image of one ring stage (32 rows x 128 B, chunk slots already swizzled).  A wave then reads one
+// contiguous 128 KB run instead of 32 rows 4 KB apart: 5.1 -> 6.1 TB/s for an empty kernel streaming this
+// workload's up-projection weights.  (Row-major weights keep working; the module tiles them when it quantises.)
+// The launch decides how many waves form a workgroup: they never synchronise.
+template <typename T, bool GLU, bool TILED>
 __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
   constexpr int KCH = 128;                       // k per ring stage
   constexpr int WR = GLU ? 2 : 1;
@@ -215,13 +221,15 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, q = lane >> 4;
-  const int expert = blockIdx.x / a.groups_per_expert;
-  const int grp = blockIdx.x - expert * a.groups_per_expert;
+  // a.groups_per_expert = wave units (CHW channels each) per expert; blockDim.x / 64 units share a workgroup
+  const int unit = blockIdx.x * (int)(blockDim.x >> 6) + wave;
+  const int expert = unit / a.groups_per_expert;
+  if (expert >= a.E) return;
   const int row_begin = expert ? a.expert_offsets[expert - 1] : 0;
   const int row_end = a.expert_offsets[expert];
   if (row_begin >= row_end) return;  // nothing routed here: the expert's weights stay untouched
-  const int n0 = (grp * 4 + wave) * CHW;
-  if (n0 >= a.N) return;             // whole wave past the last channel (waves do not synchronise)
+  const int n0 = (unit - expert * a.groups_per_expert) * CHW;
+  if (n0 >= a.N) return;             // (waves do not synchronise)
 
   unsigned char* ring = dsm + wave * DEC_WAVE_LDS;
 
@@ -245,6 +253,8 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
   }
 
   const int nst = a.K / KCH;
+  // tiled weights: this unit's K stages are consecutive 4 KB blocks
+  const unsigned char* wtile = a.wq + (size_t)unit * nst * W_BYTES + lane * 16;
   const T* __restrict__ xin = static_cast<const T*>(a.in);
   T* __restrict__ out = static_cast<T*>(a.out);
 
@@ -271,10 +281,17 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
     auto dma_stage = [&](int st, int slot) {
       const int stc = st < nst ? st : nst - 1;               // surplus rounds re-fetch the last stage
       unsigned char* dst = ring + slot * STAGE;
-      const unsigned char* wk = wexp + (size_t)stc * KCH;
+      if (TILED) {
+        const unsigned char* wk = wtile + (size_t)stc * W_BYTES;
 #pragma unroll
-      for (int j = 0; j < NWI; ++j)
-        __builtin_amdgcn_global_load_lds((glb_ptr_t)(wk + woff[j]), (lds_ptr_t)(dst + j * 1024), 16, 0, 0);
+        for (int j = 0; j < NWI; ++j)
+          __builtin_amdgcn_global_load_lds((glb_ptr_t)(wk + j * 1024), (lds_ptr_t)(dst + j * 1024), 16, 0, 0);
+      } else {
+        const unsigned char* wk = wexp + (size_t)stc * KCH;
+#pragma unroll
+        for (int j = 0; j < NWI; ++j)
+          __builtin_amdgcn_global_load_lds((glb_ptr_t)(wk + woff[j]), (lds_ptr_t)(dst + j * 1024), 16, 0, 0);
+      }
 #pragma unroll
       for (int j = 0; j < NX; ++j)
         __builtin_amdgcn_global_load_lds((glb_ptr_t)(xsrc[j] + (size_t)stc * KCH),
@@ -358,18 +375,22 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
 
 template <typename T, bool GLU>
 static int launch_decode_stream(DecodeArgs a, hipStream_t s) {
-  constexpr int CH = 4 * (GLU ? 16 : 32);
-  constexpr int LDS = 4 * DEC_WAVE_LDS;
-  auto kern = decode_fp8_stream_kernel<T, GLU>;
-  if (LDS > 64 * 1024) {
+  constexpr int CHW = GLU ? 16 : 32;
+  a.groups_per_expert = mi_ceil_div(a.N, CHW);
+  const long units = (long)a.E * a.groups_per_expert;
+  // one wave per workgroup: units are dispatched one by one as waves retire (measured 6.1 vs 5.6 TB/s for the
+  // contiguous stream with four-wave workgroups); eight fit a CU by LDS
+  const int waves = a.tiled ? 1 : 4;
+  const int lds = waves * DEC_WAVE_LDS;
+  auto kern = a.tiled ? decode_fp8_stream_kernel<T, GLU, true> : decode_fp8_stream_kernel<T, GLU, false>;
+  if (lds > 64 * 1024) {
     hipError_t e =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return (int)e;
   }
-  a.groups_per_expert = mi_ceil_div(a.N, CH);
-  long grid = (long)a.E * a.groups_per_expert;
+  const long grid = (units + waves - 1) / waves;
   if (grid > 0x7fffffffL) return MI_MOE_ESHAPE;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), LDS, s, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(waves * 64), lds, s, a);
   return mi_launch_status();
 }
 
@@ -386,7 +407,9 @@ static int launch_decode(DecodeArgs a, hipStream_t s) {
 template <typename T, bool GLU>
 static int dispatch_decode(const DecodeArgs& a, hipStream_t s) {
   // the streaming kernel needs whole 128-wide K stages and 32-bit weight offsets inside one expert
-  if (a.K % 128 == 0 && a.K >= 512 && (double)(GLU ? 2 : 1) * a.N * a.K < 4.0e9) return launch_decode_stream<T, GLU>(a, s);
+  if (a.K % 128 == 0 && (a.K >= 512 || a.tiled) && (double)(GLU ? 2 : 1) * a.N * a.K < 4.0e9)
+    return launch_decode_stream<T, GLU>(a, s);
+  if (a.tiled) return MI_MOE_EUNSUPPORTED;  // the tile layout exists for whole 128-wide K stages only
   if (a.K >= 2048) return launch_decode<T, GLU, 4>(a, s);
   if (a.K >= 1024) return launch_decode<T, GLU, 2>(a, s);
   return launch_decode<T, GLU, 1>(a, s);
@@ -405,22 +428,30 @@ static int run_decode(DecodeArgs a, int dtype, bool glu, hipStream_t s) {
   return glu ? dispatch_decode<f16_t, true>(a, s) : dispatch_decode<f16_t, false>(a, s);
 }
 
+extern "C" size_t mi_moe_fp8_tiled_bytes(int E, int N, int K, int glu) {
+  if (E < 1 || N < 1 || K < 128 || K % 128 != 0) return 0;
+  const int chw = glu ? 16 : 32;
+  return (size_t)E * mi_ceil_div(N, chw) * (size_t)(K / 128) * 4096;
+}
+
 extern "C" int mi_moe_up_swiglu_fp8(const void* x, const void* w_fc_q, const float* w_fc_scale, void* act_out,
                                     const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int H,
-                                    int I, int E, int k, int dtype, mi_moe_stream_t stream) {
+                                    int I, int E, int k, int dtype, int w_tiled, mi_moe_stream_t stream) {
   DecodeArgs a;
   a.in = x; a.wq = static_cast<const uint8_t*>(w_fc_q); a.scale = w_fc_scale; a.out = act_out;
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = H; a.N = I; a.E = E; a.kdiv = k; a.gather = 1; a.scatter = 0; a.groups_per_expert = 0;
+  a.tiled = w_tiled != 0;
   return run_decode(a, dtype, true, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mi_moe_down_fp8(const void* act, const void* w_proj_q, const float* w_proj_scale, void* o_out,
                                const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
-                               int E, int dtype, mi_moe_stream_t stream) {
+                               int E, int dtype, int w_tiled, mi_moe_stream_t stream) {
   DecodeArgs a;
   a.in = act; a.wq = static_cast<const uint8_t*>(w_proj_q); a.scale = w_proj_scale; a.out = o_out;
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = I; a.N = H; a.E = E; a.kdiv = 1; a.gather = 0; a.scatter = 1; a.groups_per_expert = 0;
+  a.tiled = w_tiled != 0;
   return run_decode(a, dtype, false, static_cast<hipStream_t>(stream));
 }

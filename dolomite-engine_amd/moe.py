@@ -72,6 +72,7 @@ class ParameterizedExperts(nn.Module):
         self.out_features = out_features
         # optional fp8 storage (see MoE.quantize_expert_weights_fp8)
         self.weight_scale_dtype = None
+        self.weight_q_glu = False
         self.register_buffer("weight_q", None, persistent=True)
         self.register_buffer("weight_scale", None, persistent=True)
         self.reset_parameters()
@@ -80,7 +81,10 @@ class ParameterizedExperts(nn.Module):
     def dense_weight(self) -> torch.Tensor:
         """The (E, out, in) weight the eager branch multiplies with (dequantised if stored as fp8)."""
         if self.weight_q is not None:
-            return (self.weight_q.float() * self.weight_scale.unsqueeze(-1)).to(self.weight_scale_dtype)
+            w_q = self.weight_q
+            if w_q.dim() == 1:  # streamed-tile layout
+                w_q = ops.fp8_untile(w_q, self.num_experts, self.out_features, self.in_features, self.weight_q_glu)
+            return (w_q.float() * self.weight_scale.unsqueeze(-1)).to(self.weight_scale_dtype)
         return self.weight
 
     def forward(self, input: torch.Tensor, num_experts_per_token: int | None = None,
@@ -124,15 +128,26 @@ class ParameterizedExperts(nn.Module):
             self.bias.zero_()
 
     @torch.no_grad()
-    def quantize_fp8(self) -> None:
+    def set_fp8_weight(self, w_q: torch.Tensor, scale: torch.Tensor, compute_dtype: torch.dtype,
+                       tiled: bool = False, glu: bool = False) -> None:
+        """Install already quantised weights: ``w_q`` (E, out, in) e4m3fn row-major, ``scale`` (E, out) fp32."""
+        if tuple(w_q.shape) != (self.num_experts, self.out_features, self.in_features) or w_q.dtype != torch.float8_e4m3fn:
+            raise ValueError("w_q must be (E, out, in) torch.float8_e4m3fn")
+        self.weight_scale_dtype = compute_dtype
+        self.weight_q_glu = glu
+        self.weight_q = ops.fp8_tile(w_q, glu) if (tiled and self.in_features % 128 == 0) else w_q
+        self.weight_scale = scale.to(torch.float32)
+        self.weight = None
+
+    @torch.no_grad()
+    def quantize_fp8(self, tiled: bool = False, glu: bool = False) -> None:
         """Replace the weight by e4m3fn values plus one fp32 scale per output channel
-        (scale = max|row| / 448)."""
+        (scale = max|row| / 448).  ``tiled`` stores the values in the layout the decode kernels stream
+        (ops.fp8_tile; ``glu`` says that the rows are [up ; gate] halves); it needs in_features % 128 == 0
+        and falls back to the row-major layout otherwise."""
         w = self.weight.detach().float()
         scale = w.abs().amax(dim=-1).clamp_min(1e-12) / 448.0
-        self.weight_scale_dtype = self.weight.dtype
-        self.weight_q = (w / scale.unsqueeze(-1)).to(torch.float8_e4m3fn)
-        self.weight_scale = scale
-        self.weight = None
+        self.set_fp8_weight((w / scale.unsqueeze(-1)).to(torch.float8_e4m3fn), scale, self.weight.dtype, tiled, glu)
 
 
 class MoE(nn.Module):
@@ -413,10 +428,12 @@ class MoE(nn.Module):
         return num_elements
 
     @torch.no_grad()
-    def quantize_expert_weights_fp8(self) -> None:
+    def quantize_expert_weights_fp8(self, tiled: bool = True) -> None:
         """Store c_fc / c_proj as e4m3fn + per-output-channel fp32 scales (decode-shape serving).
-        Not part of the reference; the eager branch then multiplies with the dequantised weights."""
+        Not part of the reference; the eager branch then multiplies with the dequantised weights.
+        ``tiled`` (default) keeps the bytes in the order the decode kernels stream them (one contiguous
+        run per wave); results do not depend on it."""
         if self.c_fc.bias is not None or self.c_proj.bias is not None:
             raise RuntimeError("fp8 expert weights do not support biases")
-        self.c_fc.quantize_fp8()
-        self.c_proj.quantize_fp8()
+        self.c_fc.quantize_fp8(tiled=tiled, glu=self._fused_swiglu)
+        self.c_proj.quantize_fp8(tiled=tiled, glu=False)

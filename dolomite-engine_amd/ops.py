@@ -290,9 +290,70 @@ def up_swiglu(x: torch.Tensor, w_fc: torch.Tensor, k: int, sorted_scattered_idxs
     return act
 
 
+def _fp8_unit_rows(glu: bool) -> int:
+    return 16 if glu else 32
+
+
+_FP8_SWIZZLE = None
+
+
+def _fp8_swizzle_index(device):
+    """(32, 1) row index and (32, 8) source-chunk index of the stage image: slot c of row t holds chunk
+    c ^ ((t >> 1) & 7)."""
+    global _FP8_SWIZZLE
+    if _FP8_SWIZZLE is None or _FP8_SWIZZLE[0].device != device:
+        t = torch.arange(32, device=device)
+        c = torch.arange(8, device=device)
+        _FP8_SWIZZLE = (t[:, None], c[None, :] ^ ((t[:, None] >> 1) & 7))
+    return _FP8_SWIZZLE
+
+
+def fp8_tile(w_q: torch.Tensor, glu: bool) -> torch.Tensor:
+    """Row-major fp8 expert weights (E, out, in) -> the streamed-tile layout of include/mi_moe.h (a flat
+    tensor): [expert][unit][K stage][32 rows][8 slots][16 bytes], units of 16 up + 16 gate channels (``glu``)
+    or 32 channels, chunk slots pre-swizzled, channels past the last one zero.  Needs in % 128 == 0."""
+    if w_q.dtype != torch.float8_e4m3fn or w_q.dim() != 3:
+        raise TypeError("expected (E, out, in) torch.float8_e4m3fn")
+    E, R, K = w_q.shape
+    if K % 128 or (glu and R % 2):
+        raise ValueError("the tile layout needs in % 128 == 0 (and an even row count for GLU weights)")
+    b = w_q.contiguous().view(torch.uint8)
+    ch = _fp8_unit_rows(glu)
+    halves = b.chunk(2, dim=1) if glu else (b,)
+    N = halves[0].shape[1]
+    U = -(-N // ch)
+    parts = []
+    for h in halves:
+        if U * ch != N:
+            h = torch.cat([h, h.new_zeros(E, U * ch - N, K)], dim=1)
+        parts.append(h.view(E, U, ch, K))
+    unit = torch.cat(parts, dim=2) if glu else parts[0]                 # (E, U, 32, K)
+    staged = unit.view(E, U, 32, K // 128, 8, 16).permute(0, 1, 3, 2, 4, 5)  # (E, U, stage, row, chunk, 16)
+    rows, src = _fp8_swizzle_index(w_q.device)
+    return staged[:, :, :, rows, src].contiguous().view(-1).view(torch.float8_e4m3fn)
+
+
+def fp8_untile(tiled: torch.Tensor, E: int, out_rows: int, K: int, glu: bool) -> torch.Tensor:
+    """Inverse of :func:`fp8_tile`: back to (E, out_rows, K) row-major."""
+    ch = _fp8_unit_rows(glu)
+    N = out_rows // 2 if glu else out_rows
+    U = -(-N // ch)
+    staged = tiled.view(torch.uint8).view(E, U, K // 128, 32, 8, 16)
+    rows, src = _fp8_swizzle_index(tiled.device)
+    unit = staged[:, :, :, rows, src].permute(0, 1, 3, 2, 4, 5).reshape(E, U, 32, K)   # the swizzle is an involution
+    if glu:
+        up = unit[:, :, :16].reshape(E, U * 16, K)[:, :N]
+        gate = unit[:, :, 16:].reshape(E, U * 16, K)[:, :N]
+        w = torch.cat([up, gate], dim=1)
+    else:
+        w = unit.reshape(E, U * 32, K)[:, :N]
+    return w.contiguous().view(torch.float8_e4m3fn)
+
+
 def up_swiglu_fp8(x: torch.Tensor, w_fc_q: torch.Tensor, w_fc_scale: torch.Tensor, k: int,
                   sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor) -> torch.Tensor:
-    """As up_swiglu with e4m3fn weights (E, 2I, H) and fp32 per-output-channel scales (E, 2I)."""
+    """As up_swiglu with e4m3fn weights and fp32 per-output-channel scales (E, 2I).  The weights are either
+    row-major (E, 2I, H) or, as a flat tensor, in the layout of :func:`fp8_tile` (``glu=True``)."""
     _dev(x, w_fc_q, w_fc_scale, sorted_scattered_idxs, expert_offsets)
     _no_grad(x)
     if w_fc_q.dtype != torch.float8_e4m3fn:
@@ -302,20 +363,29 @@ def up_swiglu_fp8(x: torch.Tensor, w_fc_q: torch.Tensor, w_fc_scale: torch.Tenso
     scale = w_fc_scale.to(torch.float32).contiguous()
     ss = _i32(sorted_scattered_idxs).contiguous()
     off = _i32(expert_offsets).contiguous()
-    E, I2, H = w_fc_q.shape
+    E, I2 = scale.shape
+    H = x.shape[1]
     L = ss.numel()
-    if x.shape[1] != H or x.shape[0] * k != L or scale.shape != (E, I2):
+    tiled = w_fc_q.dim() == 1
+    lib = _lib.load()
+    if tiled:
+        if w_fc_q.numel() != lib.mi_moe_fp8_tiled_bytes(E, I2 // 2, H, 1) or w_fc_q.numel() == 0:
+            raise ValueError("tiled weights do not match (E, 2I) scales and the hidden size of x")
+    elif tuple(w_fc_q.shape) != (E, I2, H):
+        raise ValueError("shape mismatch")
+    if x.shape[0] * k != L:
         raise ValueError("shape mismatch")
     act = torch.empty((L, I2 // 2), dtype=x.dtype, device=x.device)
     with _stage("up_swiglu_fp8"):
-        check(_lib.load().mi_moe_up_swiglu_fp8(_ptr(x), _ptr(w_fc_q), _ptr(scale), _ptr(act), _ptr(ss), _ptr(off), L, H,
-                                              I2 // 2, E, k, _code(x.dtype), _stream()))
+        check(lib.mi_moe_up_swiglu_fp8(_ptr(x), _ptr(w_fc_q), _ptr(scale), _ptr(act), _ptr(ss), _ptr(off), L, H,
+                                      I2 // 2, E, k, _code(x.dtype), int(tiled), _stream()))
     return act
 
 
 def down_fp8(act: torch.Tensor, w_proj_q: torch.Tensor, w_proj_scale: torch.Tensor,
              sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor) -> torch.Tensor:
-    """Down-projection with e4m3fn weights (E, H, I): act (L, I) grouped -> (L, H) in flat-slot order."""
+    """Down-projection with e4m3fn weights, row-major (E, H, I) or tiled (:func:`fp8_tile`, ``glu=False``):
+    act (L, I) grouped -> (L, H) in flat-slot order."""
     _dev(act, w_proj_q, w_proj_scale, sorted_scattered_idxs, expert_offsets)
     _no_grad(act)
     if w_proj_q.dtype != torch.float8_e4m3fn:
@@ -325,12 +395,19 @@ def down_fp8(act: torch.Tensor, w_proj_q: torch.Tensor, w_proj_scale: torch.Tens
     scale = w_proj_scale.to(torch.float32).contiguous()
     ss = _i32(sorted_scattered_idxs).contiguous()
     off = _i32(expert_offsets).contiguous()
-    E, H, I = w_proj_q.shape
-    L = ss.numel()
-    if act.shape != (L, I) or scale.shape != (E, H):
+    E, H = scale.shape
+    L, I = act.shape
+    tiled = w_proj_q.dim() == 1
+    lib = _lib.load()
+    if tiled:
+        if w_proj_q.numel() != lib.mi_moe_fp8_tiled_bytes(E, H, I, 0) or w_proj_q.numel() == 0:
+            raise ValueError("tiled weights do not match (E, H) scales and the width of act")
+    elif tuple(w_proj_q.shape) != (E, H, I):
+        raise ValueError("shape mismatch")
+    if ss.numel() != L:
         raise ValueError("shape mismatch")
     o = torch.empty((L, H), dtype=act.dtype, device=act.device)
     with _stage("down_fp8"):
-        check(_lib.load().mi_moe_down_fp8(_ptr(act), _ptr(w_proj_q), _ptr(scale), _ptr(o), _ptr(ss), _ptr(off), L, I, H,
-                                         E, _code(act.dtype), _stream()))
+        check(lib.mi_moe_down_fp8(_ptr(act), _ptr(w_proj_q), _ptr(scale), _ptr(o), _ptr(ss), _ptr(off), L, I, H,
+                                 E, _code(act.dtype), int(tiled), _stream()))
     return o

@@ -167,14 +167,25 @@ int mi_moe_combine_block_tail(const void* o, const void* gates, const void* shar
  * Decode-shape variants with fp8 (OCP e4m3fn) expert weights and one fp32 scale per output channel.
  * No counterpart in the reference (its fp8 support wraps nn.Linear only, lm_engine/fp8.py:63-73);
  * semantics = dequantise (w * scale[:, None]) then the two calls above.
- *   x / act / o are `dtype` (F16 / BF16); w_* are (E, out, in) bytes; *_scale are (E, out) fp32.
+ *   x / act / o are `dtype` (F16 / BF16); *_scale are (E, out) fp32.
+ *   w_tiled == 0: w_* are (E, out, in) bytes, row-major.
+ *   w_tiled == 1: w_* are in the streamed-tile layout (in % 128 == 0 only), mi_moe_fp8_tiled_bytes() bytes:
+ *       [expert][unit u][K stage s][row t = 0..31][slot c = 0..7][16 bytes]
+ *     where a unit is 16 output channels of the SwiGLU up-projection (rows t < 16: "up" channel 16u + t,
+ *     rows t >= 16: "gate" channel 16u + t - 16) or 32 channels otherwise (channel 32u + t), and slot c of
+ *     row t holds bytes [128 s + 16 c', 128 s + 16 c' + 16) of that channel's weight row with
+ *     c' = c ^ ((t >> 1) & 7).  Channels past `out` are zero rows.  A wave then streams one contiguous run
+ *     (results are bit-identical to the row-major layout; only the HBM access pattern changes).
  */
+/* out = output channels (I for the SwiGLU up-projection, whose weight has 2I rows); 0 if the layout does not
+ * exist for the shape (in % 128 != 0). */
+size_t mi_moe_fp8_tiled_bytes(int E, int out, int in, int glu);
 int mi_moe_up_swiglu_fp8(const void* x, const void* w_fc_q, const float* w_fc_scale, void* act_out,
                          const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int H, int I,
-                         int E, int k, int dtype, mi_moe_stream_t stream);
+                         int E, int k, int dtype, int w_tiled, mi_moe_stream_t stream);
 int mi_moe_down_fp8(const void* act, const void* w_proj_q, const float* w_proj_scale, void* o_out,
                     const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
-                    int E, int dtype, mi_moe_stream_t stream);
+                    int E, int dtype, int w_tiled, mi_moe_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -84,8 +84,12 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_up_swiglu(None, None, None, None, None, 16, 8, 8, 4, 2, _lib.F16, None) == E_NULL
     assert lib.mi_moe_combine(None, None, None, 4, 0, 8, _lib.BF16, None) == E_SHAPE
     assert lib.mi_moe_combine(None, None, None, 4, 2, 8, 9, None) == E_NULL  # pointers are checked before the dtype
-    assert lib.mi_moe_up_swiglu_fp8(None, None, None, None, None, None, 16, 64, 32, 4, 2, _lib.F32, None) == E_DTYPE
-    assert lib.mi_moe_down_fp8(None, None, None, None, None, None, 16, 64, 32, 4, _lib.BF16, None) == E_NULL
+    assert lib.mi_moe_up_swiglu_fp8(None, None, None, None, None, None, 16, 64, 32, 4, 2, _lib.F32, 0, None) == E_DTYPE
+    assert lib.mi_moe_down_fp8(None, None, None, None, None, None, 16, 64, 32, 4, _lib.BF16, 0, None) == E_NULL
+    assert lib.mi_moe_fp8_tiled_bytes(64, 1408, 4096, 1) == 64 * 2816 * 4096
+    assert lib.mi_moe_fp8_tiled_bytes(64, 4096, 1408, 0) == 64 * 4096 * 1408
+    assert lib.mi_moe_fp8_tiled_bytes(4, 20, 256, 1) == 4 * 2 * 2 * 4096  # 20 channels pad to two units
+    assert lib.mi_moe_fp8_tiled_bytes(4, 20, 200, 1) == 0
 
 
 def test_missing_library_fails_loudly(monkeypatch):

@@ -215,6 +215,42 @@ def test_fp8_up_down(device, dtype, T, E, k, H, I):
     torch.testing.assert_close(o.cpu().float(), ref_o, rtol=2e-2, atol=2e-3)
 
 
+@pytest.mark.parametrize("T,E,k,H,I", [(64, 64, 6, 4096, 1408), (40, 8, 2, 512, 264), (300, 4, 2, 256, 128)])
+def test_fp8_tiled_layout_is_bit_identical(device, T, E, k, H, I):
+    """The streamed-tile weight layout changes the HBM access pattern only: same bits out as row-major weights
+    (incl. a channel count that is not a multiple of the unit size, and experts with more than 16 rows).
+    With K < 512 the row-major weights run the older kernel, so there the two agree to rounding only."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(T + I)
+    se, ss, off = _routing(T, E, k, seed=3)
+    x = _rand((T, H), 1.0, torch.bfloat16, g).to(device)
+    w_fc_q, fc_scale = oracle.quantize_fp8_per_channel(torch.randn(E, 2 * I, H, generator=g) * 0.02)
+    w_pj_q, pj_scale = oracle.quantize_fp8_per_channel(torch.randn(E, H, I, generator=g) * 0.02)
+    w_fc_q, fc_scale, w_pj_q, pj_scale = (t.to(device) for t in (w_fc_q, fc_scale, w_pj_q, pj_scale))
+    ss, off = ss.to(device), off.to(device)
+    fc_t = ops.fp8_tile(w_fc_q, glu=True)
+    assert torch.equal(ops.fp8_untile(fc_t, E, 2 * I, H, True).view(torch.uint8), w_fc_q.view(torch.uint8))
+    act = ops.up_swiglu_fp8(x, w_fc_q, fc_scale, k, ss, off)
+    act_t = ops.up_swiglu_fp8(x, fc_t, fc_scale, k, ss, off)
+    if H >= 512:
+        assert torch.equal(act, act_t)
+    else:  # row-major weights with a short K take the older kernel, which sums in another order
+        torch.testing.assert_close(act_t.float(), act.float(), rtol=2e-2, atol=1e-3)
+        act = act_t
+    if I % 128 == 0:
+        pj_t = ops.fp8_tile(w_pj_q, glu=False)
+        assert torch.equal(ops.fp8_untile(pj_t, E, H, I, False).view(torch.uint8), w_pj_q.view(torch.uint8))
+        o = ops.down_fp8(act, w_pj_q, pj_scale, ss, off)
+        o_t = ops.down_fp8(act, pj_t, pj_scale, ss, off)
+        if I >= 512:
+            assert torch.equal(o, o_t)
+        else:
+            torch.testing.assert_close(o_t.float(), o.float(), rtol=2e-2, atol=1e-3)
+    else:
+        with pytest.raises(ValueError):
+            ops.fp8_tile(w_pj_q, glu=False)
+
+
 def test_fp8_all_bit_patterns(device):
     """Every e4m3fn byte value is widened exactly: K=256 one-hot activations read out each pattern."""
     ops = _ops()

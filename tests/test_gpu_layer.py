@@ -27,14 +27,10 @@ def _build(w, inputs, device, fp8=False):
             m.c_fc.weight.copy_(inputs["w_fc"])
             m.c_proj.weight.copy_(inputs["w_proj"])
     m = m.to(device).eval()
-    if fp8:
-        m.c_fc.weight = None
-        m.c_proj.weight = None
-        m.c_fc.weight_q = inputs["w_fc"].to(device)
-        m.c_fc.weight_scale = inputs["fc_scale"].to(device)
-        m.c_proj.weight_q = inputs["w_proj"].to(device)
-        m.c_proj.weight_scale = inputs["proj_scale"].to(device)
-        m.c_fc.weight_scale_dtype = m.c_proj.weight_scale_dtype = w.dtype
+    if fp8:  # in the layout the module itself chooses when it quantises (streamed tiles)
+        m.c_fc.set_fp8_weight(inputs["w_fc"].to(device), inputs["fc_scale"].to(device), w.dtype, tiled=True, glu=True)
+        m.c_proj.set_fp8_weight(inputs["w_proj"].to(device), inputs["proj_scale"].to(device), w.dtype, tiled=True,
+                                glu=False)
     if inputs["bias"] is not None:
         m.router_logit_bias = inputs["bias"].to(device)
     return m
