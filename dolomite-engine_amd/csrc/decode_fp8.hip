@@ -200,6 +200,13 @@ __device__ __forceinline__ constexpr int dec_waitcnt(int vm, int lgkm) {
 
 template <int V> struct dec_int { static constexpr int value = V; };
 
+// LDS chunk swizzles of a ring stage.  A ds_read_b128 is served in four passes of 16 lanes -- lanes
+// [8p, 8p+8) together with [16+8p, 24+8p) -- i.e. 8 consecutive rows x 2 of a lane row's chunks.  For the
+// weight rows (128 B: two rows span the 64 banks) the two chunks differ by 2, for the activation rows (256 B)
+// by 4; the XOR masks below put the 16 accesses of every pass in 16 different 16-byte bank groups.
+__device__ __forceinline__ int dec_wswz(int t) { return ((t >> 1) & 1) | (((t >> 2) & 1) << 2); }
+__device__ __forceinline__ int dec_xswz(int r) { return (r & 3) | ((r & 4) << 1); }
+
 // TILED: the weights are stored as the kernel streams them -- [expert][wave unit][K stage][4 KB], each 4 KB block
 // being the LDS image of one ring stage (32 rows x 128 B, chunk slots already swizzled).  A wave then reads one
 // contiguous 128 KB run instead of 32 rows 4 KB apart: 5.1 -> 6.1 TB/s for an empty kernel streaming this
@@ -234,7 +241,7 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
   unsigned char* ring = dsm + wave * DEC_WAVE_LDS;
 
   // weight DMA: instruction j fills ring rows [8j, 8j+8): lane -> row 8j + lane/8, slot lane%8 holding
-  // logical chunk slot ^ ((row >> 1) & 7)  (conflict-free ds_read_b128 on the 64-bank LDS)
+  // logical chunk slot ^ dec_wswz(row)
   const unsigned char* wexp = a.wq + (size_t)expert * WR * a.N * a.K;
   uint32_t woff[NWI];
 #pragma unroll
@@ -249,7 +256,7 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
       ch = n0 + t;
       if (ch > a.N - 1) ch = a.N - 1;
     }
-    woff[j] = (uint32_t)ch * (uint32_t)a.K + ((lane & 7) ^ ((t >> 1) & 7)) * 16;
+    woff[j] = (uint32_t)ch * (uint32_t)a.K + ((lane & 7) ^ dec_wswz(t)) * 16;
   }
 
   const int nst = a.K / KCH;
@@ -268,7 +275,7 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
     constexpr int NDMA = NWI + NX;
     static_assert(NS * STAGE <= DEC_WAVE_LDS, "ring does not fit");
     // activation DMA: instruction j fills ring rows [4j, 4j+4): lane -> row 4j + lane/16, slot lane%16
-    // holding logical chunk slot ^ row
+    // holding logical chunk slot ^ dec_xswz(row)
     const T* xsrc[NX];
 #pragma unroll
     for (int j = 0; j < NX; ++j) {
@@ -276,7 +283,7 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
       int srow = g0 + t;
       if (srow > row_end - 1) srow = row_end - 1;           // short pass re-reads the last row; never stored
       const int src = a.gather ? a.sorted_scattered[srow] / a.kdiv : srow;
-      xsrc[j] = xin + (size_t)src * a.K + (((lane & 15) ^ t) * 8);
+      xsrc[j] = xin + (size_t)src * a.K + (((lane & 15) ^ dec_xswz(t)) * 8);
     }
     auto dma_stage = [&](int st, int slot) {
       const int stc = st < nst ? st : nst - 1;               // surplus rounds re-fetch the last stage
@@ -313,14 +320,14 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
 #pragma unroll
       for (int m = 0; m < NM; ++m)
         xb[m] = __builtin_bit_cast(frag_t,
-                                   *reinterpret_cast<const u32x4*>(xs + xr * (KCH * 2) + (((q * NM + m) ^ xr) * 16)));
+                                   *reinterpret_cast<const u32x4*>(xs + xr * (KCH * 2) + (((q * NM + m) ^ dec_xswz(xr)) * 16)));
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
         const int t = 16 * b + r;
 #pragma unroll
         for (int h = 0; h < NM / 2; ++h) {
           const u32x4 wv =
-              *reinterpret_cast<const u32x4*>(ws + t * KCH + (((q * (NM / 2) + h) ^ ((t >> 1) & 7)) * 16));
+              *reinterpret_cast<const u32x4*>(ws + t * KCH + (((q * (NM / 2) + h) ^ dec_wswz(t)) * 16));
           acc[b] = Mfma16<T>::run(Mfma16<T>::widen(wv[0], wv[1]), xb[2 * h], acc[b]);
           acc[b] = Mfma16<T>::run(Mfma16<T>::widen(wv[2], wv[3]), xb[2 * h + 1], acc[b]);
         }

@@ -299,12 +299,12 @@ _FP8_SWIZZLE = None
 
 def _fp8_swizzle_index(device):
     """(32, 1) row index and (32, 8) source-chunk index of the stage image: slot c of row t holds chunk
-    c ^ ((t >> 1) & 7)."""
+    c ^ (((t >> 1) & 1) | (((t >> 2) & 1) << 2))."""
     global _FP8_SWIZZLE
     if _FP8_SWIZZLE is None or _FP8_SWIZZLE[0].device != device:
         t = torch.arange(32, device=device)
         c = torch.arange(8, device=device)
-        _FP8_SWIZZLE = (t[:, None], c[None, :] ^ ((t[:, None] >> 1) & 7))
+        _FP8_SWIZZLE = (t[:, None], c[None, :] ^ (((t[:, None] >> 1) & 1) | (((t[:, None] >> 2) & 1) << 2)))
     return _FP8_SWIZZLE
 
 

@@ -174,7 +174,7 @@ int mi_moe_combine_block_tail(const void* o, const void* gates, const void* shar
  *     where a unit is 16 output channels of the SwiGLU up-projection (rows t < 16: "up" channel 16u + t,
  *     rows t >= 16: "gate" channel 16u + t - 16) or 32 channels otherwise (channel 32u + t), and slot c of
  *     row t holds bytes [128 s + 16 c', 128 s + 16 c' + 16) of that channel's weight row with
- *     c' = c ^ ((t >> 1) & 7).  Channels past `out` are zero rows.  A wave then streams one contiguous run
+ *     c' = c ^ (((t >> 1) & 1) | (((t >> 2) & 1) << 2)).  Channels past `out` are zero rows.  A wave then streams one contiguous run
  *     (results are bit-identical to the row-major layout; only the HBM access pattern changes).
  */
 /* out = output channels (I for the SwiGLU up-projection, whose weight has 2I rows); 0 if the layout does not
