@@ -35,7 +35,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # from inside this process, so the figures are recorded here and are null for other workloads.
 MEASURED_TRAFFIC_BYTES = {
     "granite-3b-a800m": 1555.8e6 + 268.4e6,   # up-projection GEMM: fetch + write
-    "decode-fp8": 757.6e6 + 1.1e6,            # fp8 up-projection: fetch + write
+    "decode-fp8": 755.8e6 + 1.1e6,            # fp8 up-projection: fetch + write
 }
 
 
