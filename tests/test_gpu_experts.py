@@ -45,6 +45,8 @@ CASES = [
     (1024, 8, 2, 256, 1024),
     (700, 3, 2, 128, 260),
     (5000, 6, 3, 160, 520),   # many tiles per workgroup-list, tails in rows and columns
+    (3000, 130, 2, 128, 72),  # more than 64 experts (second chunk of the tile table), most of them nearly empty
+    (700, 250, 1, 256, 264),  # many empty experts
 ]
 
 
