@@ -147,6 +147,9 @@ def main():
     ap.add_argument("--workload", default="granite-3b-a800m")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=None)
+    ap.add_argument("--graph", action="store_true",
+                    help="also capture the forward into a HIP graph and report the time of a replay "
+                         "(ms_per_step_graph_replay); value / ms_per_step stay the eager module call")
     ap.add_argument("--fp8-row-major", action="store_true",
                     help="decode workload: keep the fp8 expert weights row-major instead of in the streamed-tile layout")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -193,6 +196,29 @@ def main():
             y = m(x)
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
+
+        graph_ms = None
+        if args.graph:
+            # the same forward captured once into a HIP graph and replayed: what a serving loop would run
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                m(x)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                y_static = m(x)
+            for _ in range(args.warmup):
+                graph.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                graph.replay()
+            torch.cuda.synchronize()
+            graph_ms = (time.perf_counter() - t0) / args.steps * 1e3
+            if not torch.equal(y_static, y):
+                print("bench.py: graph replay differs from the eager forward", file=sys.stderr)
+                sys.exit(1)
 
         # instrumented run of the same steps: HIP events around every stage
         timer = StageTimer()
@@ -243,6 +269,8 @@ def main():
         "stages_ms": stages,
         "roofline": roofline,
     }
+    if graph_ms is not None:
+        out["ms_per_step_graph_replay"] = graph_ms
     if not args.no_cpu_baseline:
         sample = args.cpu_sample_tokens or min(T, 8192)
         out["cpu_baseline"] = cpu_baseline(w, inputs, sample)
