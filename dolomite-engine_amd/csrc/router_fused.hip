@@ -210,10 +210,21 @@ __global__ __launch_bounds__(256) void router_fused_kernel(const T* __restrict__
 // With fewer than eight groups per CU the launch uses fewer waves per workgroup (so that every CU takes part)
 // and a deeper ring per wave (DEPTH 6) to keep as many bytes in flight.
 #define ROUTER_LDS_WAVES 8
-template <typename T, int DEPTH>
+// NORM folds the RMSNorm in front of the layer (ln_2 of the transformer block, mixins/dense/layer.py:58-59;
+// normalization.py:19-34 = torch.nn.RMSNorm) into the same kernel: a group's rows are streamed twice, first for
+// the sum of squares, then (out of L2) normalised as torch does -- round(x * rstd * gamma), all in fp32, one
+// rounding -- written to xnorm_out for the expert GEMMs and multiplied with the gate weights in that rounded
+// form.  The separate RMSNorm pass (read and write of (T, H)) and the router's own read of its output are gone.
+struct RouterNorm {
+  const void* gamma;  // (H,) of the model dtype, or null: no scaling
+  void* xnorm_out;    // (T, H)
+  float eps;
+};
+
+template <typename T, int DEPTH, bool NORM>
 __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ gw, const float* __restrict__ bias, int Trows, int H, int E, int k,
-    T* __restrict__ logits_out, T* __restrict__ gates, int32_t* __restrict__ idx) {
+    T* __restrict__ logits_out, T* __restrict__ gates, int32_t* __restrict__ idx, RouterNorm norm) {
   typedef typename RMfma<T>::vec frag_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char wlds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -234,8 +245,13 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
     const int kpos = step * 64 + q * 16;
     dst[0] = dst[1] = (u32x4){0u, 0u, 0u, 0u};
     if (step < nsteps && kpos < H) {  // the MFMA runs on all lanes: out-of-range k contributes zeros
-      dst[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xrow + kpos));
-      dst[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xrow + kpos + 8));
+      if (NORM) {  // read twice: keep the lines in L2
+        dst[0] = *reinterpret_cast<const u32x4*>(xrow + kpos);
+        dst[1] = *reinterpret_cast<const u32x4*>(xrow + kpos + 8);
+      } else {
+        dst[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xrow + kpos));
+        dst[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xrow + kpos + 8));
+      }
     }
   };
   auto open_group = [&](int g) {
@@ -268,6 +284,12 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
     for (int i = 0; i < 8; ++i)
       if (dst[i] >= 0) *reinterpret_cast<u32x4*>(wlds + dst[i]) = v[i];
   }
+  // NORM: gamma (or ones) as fp32 behind the weights
+  float* glds = reinterpret_cast<float*>(wlds + (size_t)E * pitch);
+  if (NORM) {
+    const T* gamma = static_cast<const T*>(norm.gamma);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) glds[i] = gamma != nullptr ? Elt<T>::load(gamma + i) : 1.0f;
+  }
   __syncthreads();
 
   const int neb = (E + 15) >> 4;
@@ -279,6 +301,38 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
     wbase[eb] = e * pitch;
   }
   while (grp < ngroups) {
+    float rstd = 1.0f;
+    if (NORM) {
+      // first pass over the group's rows: sum of squares of the 16 k this lane holds per step, then over the
+      // four lanes of the token
+      float ss = 0.f;
+      for (int s0 = 0; s0 < nsteps; s0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+          const int step = s0 + d;
+          if (step < nsteps) {
+            const u32x4 x0 = xr[d][0], x1 = xr[d][1];
+            load_x(step + DEPTH, xr[d]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float a0 = unpack_lo<T>(x0[i]), a1 = unpack_hi<T>(x0[i]);
+              const float b0 = unpack_lo<T>(x1[i]), b1 = unpack_hi<T>(x1[i]);
+              ss = fmaf(a0, a0, ss); ss = fmaf(a1, a1, ss); ss = fmaf(b0, b0, ss); ss = fmaf(b1, b1, ss);
+            }
+          }
+        }
+      }
+      ss += __shfl_xor(ss, 16, MI_WAVE);
+      ss += __shfl_xor(ss, 32, MI_WAVE);
+      rstd = 1.0f / sqrtf(ss / (float)H + norm.eps);
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) load_x(d, xr[d]);  // second pass, out of L2
+    }
+    T* xn_row = nullptr;
+    if (NORM) {
+      const int t = grp * 16 + r;
+      if (t < Trows) xn_row = static_cast<T*>(norm.xnorm_out) + (size_t)t * H;
+    }
     f32x4 acc[4];
 #pragma unroll
     for (int eb = 0; eb < 4; ++eb) acc[eb] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -289,8 +343,23 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
         if (step < nsteps) {
           const int kbyte = (step * 64 + q * 16) * (int)sizeof(T);
           const bool valid = step * 64 + q * 16 < H;
-          const u32x4 x0 = xr[d][0], x1 = xr[d][1];
+          u32x4 x0 = xr[d][0], x1 = xr[d][1];
           load_x(step + DEPTH, xr[d]);
+          if (NORM && valid) {
+            const int kpos = step * 64 + q * 16;
+            const f32x4* g4 = reinterpret_cast<const f32x4*>(glds + kpos);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const f32x4 ga = g4[i >> 1], gb = g4[2 + (i >> 1)];
+              const int o = (i & 1) * 2;
+              x0[i] = pack2<T>(unpack_lo<T>(x0[i]) * rstd * ga[o], unpack_hi<T>(x0[i]) * rstd * ga[o + 1]);
+              x1[i] = pack2<T>(unpack_lo<T>(x1[i]) * rstd * gb[o], unpack_hi<T>(x1[i]) * rstd * gb[o + 1]);
+            }
+            if (xn_row != nullptr) {
+              *reinterpret_cast<u32x4*>(xn_row + kpos) = x0;
+              *reinterpret_cast<u32x4*>(xn_row + kpos + 8) = x1;
+            }
+          }
 #pragma unroll
           for (int eb = 0; eb < 4; ++eb) {
             if (eb < neb) {
@@ -504,6 +573,26 @@ static int launch_router_splitk(const void* x, const void* gw, const float* bias
   return mi_launch_status();
 }
 
+template <typename T, bool NORM>
+static int launch_router_lds(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
+                             void* logits_out, void* gates, int32_t* idx, RouterNorm norm, size_t lds, hipStream_t s) {
+  int dev = 0, cus = 0;
+  hipError_t e;
+  if ((e = hipGetDevice(&dev)) != hipSuccess) return (int)e;
+  if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return (int)e;
+  const int groups = mi_ceil_div(T_, 16);
+  const int blocks = groups < cus ? groups : cus;
+  int waves = mi_ceil_div(groups, blocks);
+  if (waves > ROUTER_LDS_WAVES) waves = ROUTER_LDS_WAVES;
+  auto kern = waves > 4 ? router_fused_lds_kernel<T, 3, NORM> : router_fused_lds_kernel<T, 6, NORM>;
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(waves * 64), lds, s, static_cast<const T*>(x),
+                     static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out),
+                     static_cast<T*>(gates), idx, norm);
+  return mi_launch_status();
+}
+
 template <typename T>
 static int launch_router(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
                          void* logits_out, void* gates, int32_t* idx, hipStream_t s) {
@@ -516,21 +605,8 @@ static int launch_router(const void* x, const void* gw, const float* bias, int T
   // gate weights fit in LDS next to nothing else: the LDS-resident kernel
   const size_t wbytes = (size_t)E * ((size_t)H * sizeof(T) + 16);
   if (wbytes <= 156u * 1024u) {
-    int dev = 0, cus = 0;
-    hipError_t e;
-    if ((e = hipGetDevice(&dev)) != hipSuccess) return (int)e;
-    if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return (int)e;
-    const int groups = mi_ceil_div(T_, 16);
-    const int blocks = groups < cus ? groups : cus;
-    int waves = mi_ceil_div(groups, blocks);
-    if (waves > ROUTER_LDS_WAVES) waves = ROUTER_LDS_WAVES;
-    auto kern = waves > 4 ? router_fused_lds_kernel<T, 3> : router_fused_lds_kernel<T, 6>;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)wbytes);
-    if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(waves * 64), wbytes, s, static_cast<const T*>(x),
-                       static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out),
-                       static_cast<T*>(gates), idx);
-    return mi_launch_status();
+    const RouterNorm none = {nullptr, nullptr, 0.f};
+    return launch_router_lds<T, false>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, none, wbytes, s);
   }
   constexpr int TG = 2;
   dim3 grid(mi_ceil_div(T_, 4 * 16 * TG)), block(256);
@@ -565,4 +641,32 @@ extern "C" int mi_moe_router_fused(const void* x, const void* gate_w, const floa
   }
   if (dtype == MI_MOE_BF16) return launch_router<bf16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, s);
   return launch_router<f16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, s);
+}
+
+static size_t rmsnorm_router_lds_bytes(int H, int E, size_t elt) {
+  return (size_t)E * ((size_t)H * elt + 16) + (size_t)H * sizeof(float);
+}
+
+extern "C" int mi_moe_rmsnorm_router_fused_supported(int H, int E, int k, int dtype) {
+  if (H < 1 || E < 1 || E > 64 || k < 1 || k > ROUTER_KMAX || k > E || H % 16 != 0) return 0;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return 0;
+  return rmsnorm_router_lds_bytes(H, E, 2) <= 156u * 1024u;
+}
+
+extern "C" int mi_moe_rmsnorm_router_fused(const void* h, const void* ln_weight, float eps, const void* gate_w,
+                                           const float* bias, int T, int H, int E, int k, int dtype,
+                                           void* x_norm_out, void* logits_out, void* gates_out, int32_t* idx_out,
+                                           mi_moe_stream_t stream) {
+  if (T < 0 || H < 1 || E < 1 || k < 1 || k > E) return MI_MOE_ESHAPE;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (!mi_moe_rmsnorm_router_fused_supported(H, E, k, dtype)) return MI_MOE_EUNSUPPORTED;
+  if (T == 0) return MI_MOE_OK;
+  if (!h || !gate_w || !x_norm_out || !gates_out || !idx_out) return MI_MOE_ENULL;
+  if (!mi_aligned(h, 16) || !mi_aligned(gate_w, 16) || !mi_aligned(x_norm_out, 16)) return MI_MOE_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const RouterNorm norm = {ln_weight, x_norm_out, eps};
+  const size_t lds = rmsnorm_router_lds_bytes(H, E, 2);
+  if (dtype == MI_MOE_BF16)
+    return launch_router_lds<bf16_t, true>(h, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, norm, lds, s);
+  return launch_router_lds<f16_t, true>(h, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, norm, lds, s);
 }

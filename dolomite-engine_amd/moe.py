@@ -216,11 +216,15 @@ class MoE(nn.Module):
     # ---------------------------------------------------------------------------------------------
 
     def forward(self, hidden_states: torch.Tensor, residual: torch.Tensor | None = None,
-                residual_scale: float | None = None) -> torch.Tensor:
-        """moe.py:212-244.  ``residual`` / ``residual_scale`` are an extension: with them the result is
-        ``moe(hidden_states) * residual_scale + residual``, i.e. the two lines the transformer block runs after
-        its mlp_block (mixins/dense/layer.py:61-66); on the kernel branch they -- and the shared-expert sum --
-        are folded into the combine pass, with the roundings of the separate operations."""
+                residual_scale: float | None = None, pre_norm: tuple | None = None) -> torch.Tensor:
+        """moe.py:212-244.  Extensions that take in the block's code around the layer
+        (mixins/dense/layer.py:58-66):
+
+        * ``pre_norm = (weight or None, eps)``: ``hidden_states`` is first RMS-normalised (the block's ``ln_2``);
+          on the kernel branch the normalisation runs inside the router kernel;
+        * ``residual`` / ``residual_scale``: the result is ``moe(...) * residual_scale + residual``; on the kernel
+          branch they -- and the shared-expert sum -- are folded into the combine pass, with the roundings of the
+          separate operations."""
         if not self.use_padding_free_transformer:
             batch_size, sequence_length, _ = hidden_states.shape
 
@@ -228,7 +232,22 @@ class MoE(nn.Module):
         if residual is not None:
             residual = residual.reshape(-1, self.hidden_size)
 
-        router_logits, router_weights, selected_experts = self._compute_routing_weights(hidden_states)
+        routed = None
+        if pre_norm is not None:
+            norm_weight, norm_eps = pre_norm
+            if self._use_fused_router(hidden_states) and ops.rmsnorm_router_fused_supported(
+                hidden_states, self.num_experts, self.top_k
+            ):
+                hidden_states, _, router_weights, selected_experts = ops.rmsnorm_router_fused(
+                    hidden_states, norm_weight, norm_eps, self.gate.weight, self.top_k, bias=self.router_logit_bias
+                )
+                routed = (None, router_weights, selected_experts)
+            else:
+                hidden_states = F.rms_norm(hidden_states, (self.hidden_size,), norm_weight, norm_eps)
+
+        router_logits, router_weights, selected_experts = (
+            routed if routed is not None else self._compute_routing_weights(hidden_states)
+        )
 
         # the tail can only be folded in where nothing sits between the expert sum and it
         fuse_tail = (

@@ -151,6 +151,42 @@ def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch
     return logits, gates, idx
 
 
+def rmsnorm_router_fused_supported(x: torch.Tensor, num_experts: int, k: int) -> bool:
+    return (x.dtype in (torch.bfloat16, torch.float16) and x.is_cuda
+            and bool(_lib.load().mi_moe_rmsnorm_router_fused_supported(x.shape[-1], num_experts, k, _code(x.dtype))))
+
+
+def rmsnorm_router_fused(h: torch.Tensor, ln_weight: torch.Tensor | None, eps: float, gate_weight: torch.Tensor,
+                         k: int, bias: torch.Tensor | None = None, return_logits: bool = False):
+    """RMSNorm (torch.nn.RMSNorm semantics: fp32 arithmetic, one rounding) + fused router in one kernel.
+
+    Stands in for ``ln_2`` followed by the routing of the layer (mixins/dense/layer.py:58-59, moe.py:246-257).
+    Returns (x_norm (T, H), logits or None, gates (T, k), experts (T, k) int32)."""
+    _dev(h, ln_weight, gate_weight, bias)
+    _no_grad(h, gate_weight)
+    h = h.contiguous()
+    gate_weight = gate_weight.contiguous()
+    T, H = h.shape
+    E = gate_weight.shape[0]
+    if gate_weight.dtype != h.dtype or gate_weight.shape[1] != H:
+        raise ValueError("gate weight must be (E, H) in the dtype of h")
+    if ln_weight is not None:
+        if ln_weight.shape != (H,):
+            raise ValueError("ln_weight must be (H,)")
+        ln_weight = ln_weight.to(h.dtype).contiguous()
+    if bias is not None:
+        bias = bias.to(torch.float32).contiguous()
+    x_norm = torch.empty_like(h)
+    logits = torch.empty((T, E), dtype=h.dtype, device=h.device) if return_logits else None
+    gates = torch.empty((T, k), dtype=h.dtype, device=h.device)
+    idx = torch.empty((T, k), dtype=torch.int32, device=h.device)
+    with _stage("rmsnorm_router_fused"):
+        check(_lib.load().mi_moe_rmsnorm_router_fused(_ptr(h), _ptr(ln_weight), float(eps), _ptr(gate_weight), _ptr(bias),
+                                                     T, H, E, k, _code(h.dtype), _ptr(x_norm), _ptr(logits),
+                                                     _ptr(gates), _ptr(idx), _stream()))
+    return x_norm, logits, gates, idx
+
+
 def continuous_count(x: torch.Tensor, size: int) -> torch.Tensor:
     """Histogram of the integer tensor ``x`` with ``size`` bins, uint32 (moe.py:38-44)."""
     _dev(x)

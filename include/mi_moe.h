@@ -82,6 +82,21 @@ int mi_moe_router_fused(const void* x, const void* gate_w, const float* bias, in
                         size_t ws_bytes, mi_moe_stream_t stream);
 
 /*
+ * RMSNorm + fused router: x_norm = round(h * rsqrt(mean(h^2) + eps) * ln_weight) (computed in fp32, one rounding,
+ * as torch.nn.RMSNorm does), written to x_norm_out, then the fused router above on x_norm -- in one kernel.
+ * Replaces: ln_2 of the transformer block followed by MoE._compute_routing_weights
+ * (mixins/dense/layer.py:58-59, normalization.py:19-34, moe.py:246-257).
+ *   h (T, H), ln_weight (H,) of `dtype` or NULL (no scaling), x_norm_out (T, H).
+ * The gate weights and ln_weight must fit in LDS: mi_moe_rmsnorm_router_fused_supported() says whether the shape
+ * is taken (E * (2H + 16) + 4H <= 156 KiB, E <= 64, k <= 8, H % 16 == 0, F16 / BF16); otherwise
+ * MI_MOE_EUNSUPPORTED and the caller runs the two steps separately.
+ */
+int mi_moe_rmsnorm_router_fused_supported(int H, int E, int k, int dtype);
+int mi_moe_rmsnorm_router_fused(const void* h, const void* ln_weight, float eps, const void* gate_w,
+                                const float* bias, int T, int H, int E, int k, int dtype, void* x_norm_out,
+                                void* logits_out, void* gates_out, int32_t* idx_out, mi_moe_stream_t stream);
+
+/*
  * Histogram of expert ids.
  * Replaces: continuous_count_cute / the bincount custom op (moe.py:27-44).
  *   ids (L,) int32 with values in [0, E); counts_out (E,) uint32.  1 <= E <= 1024.

@@ -257,6 +257,16 @@ def moe_forward(x: torch.Tensor, gate_weight: torch.Tensor, w_fc: torch.Tensor, 
     return OracleOutput(y, logits, gates, experts, se, ss, off)
 
 
+def rmsnorm(h: torch.Tensor, weight: torch.Tensor | None, eps: float) -> torch.Tensor:
+    """torch.nn.RMSNorm as the reference's RMSNorm falls back to (normalization.py:19-34): fp32 arithmetic,
+    x * rsqrt(mean(x^2) + eps) * weight, one rounding to the input dtype."""
+    hf = h.float()
+    y = hf * torch.rsqrt(hf.pow(2).mean(-1, keepdim=True) + eps)
+    if weight is not None:
+        y = y * weight.float()
+    return y.to(h.dtype)
+
+
 def switch_aux_loss(logits: torch.Tensor, selected_experts: torch.Tensor) -> torch.Tensor:
     """moe.py:346-369 without the data-parallel all-reduce (single process)."""
     logits = logits.view(-1, logits.size(-1))

@@ -164,6 +164,32 @@ def test_layer_block_tail(device, dtype, shared_size):
     torch.testing.assert_close(eager.float(), fused.float(), rtol=2e-2, atol=2e-2)
 
 
+def test_layer_with_pre_norm(device):
+    """ln_2 folded into the layer: same routing and (to rounding of x_norm) same output as RMSNorm followed by the
+    layer, on the kernel branch and on the eager branch; and close to the fp32 oracle of norm + layer."""
+    from dolomite_engine_amd import Kernel, MoE, enable_kernels
+
+    torch.manual_seed(3)
+    m = MoE(hidden_size=256, intermediate_size=128, shared_intermediate_size=None, num_experts=8,
+            num_experts_per_tok=2, activation_function="swiglu", add_bias=False, dropout=0.0, init_method="normal",
+            initializer_range=0.05, m_width=None, num_layers=1, use_padding_free_transformer=True)
+    m = m.to(torch.bfloat16).to(device).eval()
+    h = (torch.randn(777, 256, device=device) * 3).bfloat16()
+    lnw = (1 + 0.2 * torch.randn(256, device=device)).bfloat16()
+    res = torch.randn(777, 256, device=device).bfloat16()
+    with torch.no_grad(), enable_kernels([Kernel.scattermoe]):
+        fused = m(h, residual=res, residual_scale=0.5, pre_norm=(lnw, 1e-5))
+        unfused = m(torch.nn.functional.rms_norm(h, (256,), lnw, 1e-5), residual=res, residual_scale=0.5)
+    with torch.no_grad():
+        eager = m(h, residual=res, residual_scale=0.5, pre_norm=(lnw, 1e-5))
+    torch.testing.assert_close(fused.float(), unfused.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(fused.float(), eager.float(), rtol=2e-2, atol=2e-2)
+    xn = oracle.rmsnorm(h.cpu(), lnw.cpu(), 1e-5)
+    ref = oracle.moe_forward(xn, m.gate.weight.cpu(), m.c_fc.weight.cpu(), m.c_proj.weight.cpu(), 2,
+                             residual=res.cpu(), residual_scale=0.5)
+    torch.testing.assert_close(fused.cpu().float(), ref.y, rtol=2e-2, atol=2e-2)
+
+
 def test_combine_block_tail_matches_separate_ops(device):
     """mi_moe_combine_block_tail == mi_moe_combine followed by torch's add / mul / add, bit for bit, for
     every subset of the three optional steps (vector and scalar kernels)."""

@@ -137,3 +137,49 @@ def test_router_fused(device, dtype, T, H, E, k, bias):
     assert torch.equal(idx3.cpu().long(), ref_idx3)
     ulp3 = (gates3.cpu().view(torch.int16).int() - oracle.softmax_topk(vals3, dtype).view(torch.int16).int()).abs().max()
     assert ulp3 <= 1
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E,k,bias,gamma", [(1, 64, 8, 2, False, True), (200, 256, 40, 8, True, True),
+                                                (2500, 1536, 40, 8, True, True), (4099, 1024, 32, 8, False, False),
+                                                (333, 48, 5, 1, False, True)])
+def test_rmsnorm_router_fused(device, dtype, T, H, E, k, bias, gamma):
+    """RMSNorm folded into the router kernel: x_norm equals the oracle's RMSNorm up to one unit in the last place
+    (the sum of squares is added in another order), and everything after it is the fused router's contract on the
+    device's own x_norm."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(T + H + E)
+    h = (torch.randn(T, H, generator=g) * 2.5).to(dtype)
+    lnw = (1 + 0.2 * torch.randn(H, generator=g)).to(dtype) if gamma else None
+    w = (torch.randn(E, H, generator=g) * 0.02).to(dtype)
+    b = (torch.randn(E, generator=g) * 0.5) if bias else None
+    assert ops.rmsnorm_router_fused_supported(h.to(device), E, k)
+    print(f"rmsnorm_router_fused T={T} H={H} E={E} k={k} {dtype}", flush=True)
+    x_norm, logits, gates, idx = ops.rmsnorm_router_fused(
+        h.to(device), None if lnw is None else lnw.to(device), 1e-5, w.to(device), k,
+        bias=None if b is None else b.to(device), return_logits=True)
+    ref_norm = oracle.rmsnorm(h, lnw, 1e-5)
+    bits = torch.int16
+    ulp = (x_norm.cpu().view(bits).int() - ref_norm.view(bits).int()).abs()
+    assert ulp.max() <= 1 and (ulp > 0).float().mean() < 1e-3
+    # from here on: the fused router on the device's x_norm
+    xn = x_norm.cpu()
+    ref_logits = oracle.router_logits(xn, w, b)
+    torch.testing.assert_close(logits.cpu().float(), ref_logits.float(), rtol=1.6e-2 if dtype == torch.bfloat16 else 2e-3,
+                               atol=1e-3)
+    vals, ref_idx = oracle.topk_canonical(logits.cpu(), k)
+    assert torch.equal(idx.cpu().long(), ref_idx)
+    ref_gates = oracle.softmax_topk(vals, dtype)
+    assert (gates.cpu().view(bits).int() - ref_gates.view(bits).int()).abs().max() <= 1
+    # and the unfused pair of calls on that x_norm gives the same routing
+    logits2, gates2, idx2 = ops.router_fused(x_norm, w.to(device), k, bias=None if b is None else b.to(device),
+                                             return_logits=True)
+    torch.testing.assert_close(logits2.float(), logits.float(), rtol=1.6e-2 if dtype == torch.bfloat16 else 2e-3, atol=1e-3)
+
+
+def test_rmsnorm_router_fused_unsupported_shapes(device):
+    ops = _ops()
+    x = torch.zeros(4, 4096, dtype=torch.bfloat16, device=device)
+    assert not ops.rmsnorm_router_fused_supported(x, 64, 6)       # 64 x 4096 gate weights do not fit in LDS
+    assert ops.rmsnorm_router_fused_supported(x, 8, 2)
+    assert not ops.rmsnorm_router_fused_supported(x.float(), 8, 2)

@@ -358,3 +358,22 @@ def test_zipf_bias_skews_the_load():
     assert abs(first.max().item() - p_max) < 0.05 * p_max + 0.01  # top-1 share follows Zipf(1.1)
     load = torch.bincount(logits.topk(w.k, -1).indices.flatten(), minlength=w.E).double()
     assert load.max() / load.min() > 8  # slot counts differ by about an order of magnitude
+
+
+def test_rmsnorm_equals_torch_module_and_closed_form():
+    """oracle.rmsnorm is pinned by torch.nn.RMSNorm itself (the class the reference subclasses,
+    normalization.py:19) bit for bit in bf16 / fp16 / fp32, and by a closed form: rows of constant magnitude c
+    normalise to sign(x) * weight (up to eps)."""
+    g = torch.Generator().manual_seed(2)
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        x = (torch.randn(37, 96, generator=g) * 1.7).to(dtype)
+        w = (1 + 0.1 * torch.randn(96, generator=g)).to(dtype)
+        m = torch.nn.RMSNorm(96, eps=1e-5).to(dtype)
+        with torch.no_grad():
+            m.weight.copy_(w)
+            want = m(x)
+        assert torch.equal(oracle.rmsnorm(x, w, 1e-5), want), dtype
+        assert torch.equal(oracle.rmsnorm(x, None, 1e-5), torch.nn.functional.rms_norm(x, (96,), None, 1e-5)), dtype
+    s = torch.where(torch.rand(5, 64, generator=g) < 0.5, -3.0, 3.0)
+    w = torch.linspace(0.5, 2.0, 64)
+    torch.testing.assert_close(oracle.rmsnorm(s, w, 0.0), torch.sign(s) * w, rtol=1e-6, atol=1e-6)
