@@ -1,0 +1,88 @@
+"""Training through the kernel branch: the expert computation as a differentiable function.
+
+The forward is the same three launches as in inference (up-projection with fused SwiGLU, down-projection,
+combine).  The backward reuses the grouped GEMM for everything that is a "rows times expert weight" product --
+the gradient w.r.t. the activations of both projections and the recomputation of the two intermediates that
+are not kept -- and leaves the per-expert weight gradients (X^T dY per expert, a contraction over the rows) to
+one library GEMM per expert.  The reference gets both from the external scattermoe autograd function
+(lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:91-101); this module is the counterpart for the
+gradient, built on this package's forward kernels.
+
+Memory kept for the backward: x, the gates, the routing indices and the (L, I) activation; the (L, 2I)
+pre-activation and the (L, H) expert outputs are recomputed.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+
+class ScatteredSwiGLUExperts(torch.autograd.Function):
+    """y[t] = sum_j gates[t, j] * ( swiglu(x[t] @ w_fc[e]^T) @ w_proj[e]^T ),  e = expert of slot (t, j)."""
+
+    @staticmethod
+    def forward(ctx, x, w_fc, w_proj, gates, sorted_scattered, expert_offsets, k):
+        act = ops.up_swiglu(x, w_fc, k, sorted_scattered, expert_offsets)
+        o = ops.scattered_gemm(act, w_proj, 1, sorted_scattered, expert_offsets, True, False)
+        y = ops.combine(o, gates)
+        ctx.save_for_backward(x, w_fc, w_proj, gates, sorted_scattered, expert_offsets, act)
+        ctx.k = k
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w_fc, w_proj, gates, ss, off, act = ctx.saved_tensors
+        k = ctx.k
+        T, H = x.shape
+        E, I2, _ = w_fc.shape
+        I = I2 // 2
+        dy = dy.contiguous()
+        ssl = ss.long()
+        tok = ssl // k                                # token of every sorted row
+        g_sorted = gates.reshape(-1)[ssl]             # gate of every sorted row
+
+        half = x.dtype in (torch.float16, torch.bfloat16)
+
+        # gradient w.r.t. the gates: <dy[t], o[t, j]>, o recomputed from the kept activation
+        o = ops.scattered_gemm(act, w_proj, 1, ss, off, True, False)
+        if half and H % 8 == 0:
+            d_gates = ops.combine_grad_gates(o, dy, k)
+        else:
+            d_gates = torch.bmm(o.view(T, k, H), dy.unsqueeze(-1)).squeeze(-1)
+        del o
+
+        # gradient w.r.t. the SwiGLU output, in grouped order: dy[t_i] @ w_proj[e_i]; the gate g_i of the row
+        # is applied together with the SwiGLU backward on the recomputed pre-activation
+        d_act = ops.scattered_gemm(dy, w_proj.transpose(1, 2).contiguous(), k, ss, off, False, True)
+        h = ops.scattered_gemm(x, w_fc, k, ss, off, False, True)
+        if half and I % 8 == 0:
+            d_h = ops.swiglu_backward(h, d_act, g_sorted)
+        else:
+            up, gate = h[:, :I].float(), h[:, I:].float()
+            sig = torch.sigmoid(gate)
+            da = d_act.float() * g_sorted.float().unsqueeze(-1)
+            d_h = torch.cat([da * gate * sig, da * up * sig * (1.0 + gate * (1.0 - sig))], dim=1).to(x.dtype)
+            del up, gate, sig, da
+        del h, d_act
+
+        # gradient w.r.t. x: every slot's contribution in flat-slot order, then the k slots of a token summed
+        dx_slots = ops.scattered_gemm(d_h, w_fc.transpose(1, 2).contiguous(), 1, ss, off, True, False)
+        dx = dx_slots.view(T, k, H).sum(dim=1)
+        del dx_slots
+
+        # weight gradients: per expert X^T dY over that expert's rows
+        d_w_fc = torch.zeros_like(w_fc)
+        d_w_proj = torch.zeros_like(w_proj)
+        act_g = act * g_sorted.unsqueeze(-1)          # (g dy)^T a == dy^T (g a), and a is the narrower of the two
+        ends = off.tolist()
+        start = 0
+        for e, end in enumerate(ends):
+            if end > start:
+                rows = slice(start, end)
+                t_e = tok[rows]
+                d_w_fc[e] = d_h[rows].t() @ x[t_e]
+                d_w_proj[e] = dy[t_e].t() @ act_g[rows]
+            start = end
+        return dx, d_w_fc, d_w_proj, d_gates.to(gates.dtype), None, None, None

@@ -27,6 +27,7 @@ import torch.nn.functional as F
 
 from . import ops
 from .activations import GLUActivation, get_activation_function, is_glu
+from .autograd import ScatteredSwiGLUExperts
 from .enums import Kernel
 from .kernels import is_kernel_allowed
 from .linear import ParameterizedLinear
@@ -252,6 +253,7 @@ class MoE(nn.Module):
         # the tail can only be folded in where nothing sits between the expert sum and it
         fuse_tail = (
             is_kernel_allowed(Kernel.scattermoe)
+            and not self._needs_grad(hidden_states)
             and isinstance(self.dropout, nn.Identity)
             and (self.shared_intermediate_size is not None or residual is not None or residual_scale is not None)
         )
@@ -289,10 +291,16 @@ class MoE(nn.Module):
 
         return hidden_states
 
+    def _needs_grad(self, hidden_states: torch.Tensor) -> bool:
+        return torch.is_grad_enabled() and (
+            hidden_states.requires_grad or any(p.requires_grad for p in self.parameters())
+        )
+
     def _use_fused_router(self, hidden_states: torch.Tensor) -> bool:
         return (
             is_kernel_allowed(Kernel.scattermoe)
             and not self.training
+            and not self._needs_grad(hidden_states)
             and hidden_states.is_cuda
             and ops.router_fused_supported(hidden_states, self.num_experts, self.top_k)
         )
@@ -326,7 +334,14 @@ class MoE(nn.Module):
             shared, residual, residual_scale = tail if tail is not None else (None, None, None)
             sorted_expert_idxs, sorted_scattered_idxs, expert_offsets = ops.sort_bin(selected_experts, self.num_experts)
 
-            if self.c_fc.weight_q is not None:
+            if self.c_fc.weight_q is None and self._fused_swiglu and self._needs_grad(hidden_states):
+                # training: the same forward kernels inside a differentiable function (autograd.py)
+                assert self.c_fc.bias is None and tail is None
+                hidden_states = ScatteredSwiGLUExperts.apply(
+                    hidden_states, self.c_fc.weight, self.c_proj.weight, router_weights, sorted_scattered_idxs,
+                    expert_offsets, self.top_k
+                )
+            elif self.c_fc.weight_q is not None:
                 if not self._fused_swiglu:
                     raise RuntimeError("fp8 expert weights need the swiglu activation")
                 hidden_states = ops.up_swiglu_fp8(hidden_states, self.c_fc.weight_q, self.c_fc.weight_scale,

@@ -281,6 +281,43 @@ def combine(o: torch.Tensor, gates: torch.Tensor, shared: torch.Tensor | None = 
     return y
 
 
+def swiglu_backward(h: torch.Tensor, d_act: torch.Tensor, row_scale: torch.Tensor | None = None) -> torch.Tensor:
+    """Gradient of ``a = h[:, :I] * silu(h[:, I:])`` (activations/glu.py:42-43) w.r.t. ``h`` given ``d_act``
+    (L, I); ``row_scale`` (L,) multiplies ``d_act`` per row first.  16-bit dtypes."""
+    _dev(h, d_act, row_scale)
+    _no_grad(h, d_act)
+    h = h.contiguous()
+    d_act = d_act.contiguous()
+    L, I = d_act.shape
+    if tuple(h.shape) != (L, 2 * I) or h.dtype != d_act.dtype:
+        raise ValueError("h must be (L, 2I) and d_act (L, I) of the same dtype")
+    if row_scale is not None:
+        row_scale = row_scale.contiguous()
+        if tuple(row_scale.shape) != (L,) or row_scale.dtype != h.dtype:
+            raise ValueError("row_scale must be (L,) in the dtype of h")
+    d_h = torch.empty_like(h)
+    with _stage("swiglu_backward"):
+        check(_lib.load().mi_moe_swiglu_backward(_ptr(h), _ptr(d_act), _ptr(row_scale), _ptr(d_h), L, I,
+                                                 _code(h.dtype), _stream()))
+    return d_h
+
+
+def combine_grad_gates(o: torch.Tensor, dy: torch.Tensor, k: int) -> torch.Tensor:
+    """d_gates[t, j] = <dy[t], o[t*k + j]>: the gradient of :func:`combine` w.r.t. the gates.  16-bit dtypes."""
+    _dev(o, dy)
+    _no_grad(o, dy)
+    o = o.contiguous()
+    dy = dy.contiguous()
+    T, H = dy.shape
+    if tuple(o.shape) != (T * k, H) or o.dtype != dy.dtype:
+        raise ValueError("o must be (T*k, H) and dy (T, H) of the same dtype")
+    d_gates = torch.empty((T, k), dtype=o.dtype, device=o.device)
+    with _stage("combine_grad_gates"):
+        check(_lib.load().mi_moe_combine_grad_gates(_ptr(o), _ptr(dy), _ptr(d_gates), T, k, H, _code(o.dtype),
+                                                    _stream()))
+    return d_gates
+
+
 def scattered_experts(inputs: torch.Tensor, expert_weights: torch.Tensor, k: int,
                       sorted_expert_idxs: torch.Tensor, sorted_scattered_idxs: torch.Tensor,
                       expert_offsets: torch.Tensor, gates: torch.Tensor | None = None, grouped_in: bool = False,

@@ -179,6 +179,21 @@ int mi_moe_combine_block_tail(const void* o, const void* gates, const void* shar
                               mi_moe_stream_t stream);
 
 /*
+ * Element-wise pieces of the backward pass (training through the kernel branch).  The reference gets its
+ * gradients from the autograd function of the external scattermoe package (moe.py:91-101); these two are
+ * the parts of that backward that are neither a grouped GEMM nor a library GEMM.  F16 / BF16 only.
+ *
+ * mi_moe_swiglu_backward: h (L, 2I) = [up | gate] pre-activation, d_act (L, I) gradient of up * silu(gate)
+ * (activations/glu.py:42-43), row_scale (L,) or NULL (a factor on d_act per row: the gate weight of the
+ * row's slot), d_h (L, 2I) out = [d_act * silu(gate) | d_act * up * silu'(gate)].  I % 8 == 0.
+ */
+int mi_moe_swiglu_backward(const void* h, const void* d_act, const void* row_scale, void* d_h, int L, int I,
+                           int dtype, mi_moe_stream_t stream);
+/* d_gates[t, j] = <dy[t, :], o[t*k + j, :]>: the gradient of mi_moe_combine w.r.t. the gates.  H % 8 == 0. */
+int mi_moe_combine_grad_gates(const void* o, const void* dy, void* d_gates, int T, int k, int H, int dtype,
+                              mi_moe_stream_t stream);
+
+/*
  * Decode-shape variants with fp8 (OCP e4m3fn) expert weights and one fp32 scale per output channel.
  * No counterpart in the reference (its fp8 support wraps nn.Linear only, lm_engine/fp8.py:63-73);
  * semantics = dequantise (w * scale[:, None]) then the two calls above.

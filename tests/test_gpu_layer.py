@@ -249,17 +249,61 @@ def test_layer_under_hip_graph_capture(device, name, T):
             assert torch.equal(static_y, eager), f"replay {i}"
 
 
-def test_kernel_branch_refuses_grad(device):
+def test_kernel_branch_refuses_grad_without_swiglu(device):
+    """Only the SwiGLU path has a backward; other activations on the kernel branch stay forward-only and say so."""
     from dolomite_engine_amd import Kernel, MoE, enable_kernels
 
     m = MoE(hidden_size=64, intermediate_size=64, shared_intermediate_size=None, num_experts=4,
-            num_experts_per_tok=2, activation_function="swiglu", add_bias=False, dropout=0.0, init_method="normal",
-            initializer_range=0.02, m_width=None, num_layers=1, use_padding_free_transformer=True)
+            num_experts_per_tok=2, activation_function="gelu_pytorch_tanh", add_bias=False, dropout=0.0,
+            init_method="normal", initializer_range=0.02, m_width=None, num_layers=1,
+            use_padding_free_transformer=True)
     m = m.to(torch.bfloat16).to(device).eval()
     x = torch.randn(8, 64, device=device, dtype=torch.bfloat16)
     with enable_kernels([Kernel.scattermoe]):
         with pytest.raises(RuntimeError, match="forward-only"):
             m(x)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, dict(rtol=2e-3, atol=2e-5)), (torch.bfloat16, dict(rtol=5e-2, atol=2e-2))])
+@pytest.mark.parametrize("shared", [None, 64])
+def test_training_gradients_match_eager_branch(device, dtype, tol, shared):
+    """Training through the kernel branch: output, aux loss and every gradient (input, router, both expert
+    weight tensors, shared experts) against torch autograd through the eager branch of the same module."""
+    from dolomite_engine_amd import Kernel, MoE, enable_kernels
+    from dolomite_engine_amd.loss import clear_aux_loss, get_aux_loss
+
+    torch.manual_seed(21)
+    m = MoE(hidden_size=128, intermediate_size=64, shared_intermediate_size=shared, num_experts=8,
+            num_experts_per_tok=2, activation_function="swiglu", add_bias=False, dropout=0.0, init_method="normal",
+            initializer_range=0.1, m_width=None, num_layers=1, use_padding_free_transformer=True)
+    m = m.to(dtype).to(device).train()
+    x0 = torch.randn(300, 128, device=device, dtype=dtype)
+    dy = torch.randn(300, 128, device=device, dtype=dtype)
+
+    def run(kernels):
+        m.zero_grad(set_to_none=True)
+        clear_aux_loss()
+        x = x0.clone().requires_grad_(True)
+        if kernels:
+            with enable_kernels([Kernel.scattermoe]):
+                y = m(x)
+        else:
+            y = m(x)
+        aux = get_aux_loss()
+        ((y * dy).sum() + 0.01 * aux).backward()
+        grads = {n: p.grad.detach().clone() for n, p in m.named_parameters()}
+        return y.detach(), aux.detach(), x.grad.detach(), grads
+
+    y_e, aux_e, dx_e, g_e = run(False)
+    y_k, aux_k, dx_k, g_k = run(True)
+    torch.testing.assert_close(y_k.float(), y_e.float(), **tol)
+    torch.testing.assert_close(aux_k.float(), aux_e.float(), rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(dx_k.float(), dx_e.float(), **tol)
+    assert set(g_k) == set(g_e)
+    for n in g_e:
+        scale = g_e[n].float().abs().max().clamp_min(1e-6)
+        # relative to the largest entry of the gradient: both branches round bf16 intermediates differently
+        torch.testing.assert_close(g_k[n].float() / scale, g_e[n].float() / scale, rtol=tol["rtol"], atol=tol["rtol"]), n
 
 
 @pytest.mark.parametrize("name", ["granite-1b-a400m", "granite-3b-a800m", "mixtral"])
