@@ -3,8 +3,8 @@
 The forward is the same three launches as in inference (up-projection with fused SwiGLU, down-projection,
 combine).  The backward reuses the grouped GEMM for everything that is a "rows times expert weight" product --
 the gradient w.r.t. the activations of both projections and the recomputation of the two intermediates that
-are not kept -- and leaves the per-expert weight gradients (X^T dY per expert, a contraction over the rows) to
-one library GEMM per expert.  The reference gets both from the external scattermoe autograd function
+are not kept -- and a second kernel, a grouped X^T dY contracted over each expert's rows, for the weight
+gradients (fp32 and odd shapes fall back to one library GEMM per expert).  The reference gets both from the external scattermoe autograd function
 (lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:91-101); this module is the counterpart for the
 gradient, built on this package's forward kernels.
 
@@ -73,16 +73,20 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
         del dx_slots
 
         # weight gradients: per expert X^T dY over that expert's rows
-        d_w_fc = torch.zeros_like(w_fc)
-        d_w_proj = torch.zeros_like(w_proj)
         act_g = act * g_sorted.unsqueeze(-1)          # (g dy)^T a == dy^T (g a), and a is the narrower of the two
-        ends = off.tolist()
-        start = 0
-        for e, end in enumerate(ends):
-            if end > start:
-                rows = slice(start, end)
-                t_e = tok[rows]
-                d_w_fc[e] = d_h[rows].t() @ x[t_e]
-                d_w_proj[e] = dy[t_e].t() @ act_g[rows]
-            start = end
+        if half and ops.grouped_wgrad_supported(d_h, x, E):
+            tok32 = tok.to(torch.int32)
+            d_w_fc = ops.grouped_wgrad(d_h, x, off, None, tok32)
+            d_w_proj = ops.grouped_wgrad(dy, act_g, off, tok32, None)
+        else:
+            d_w_fc = torch.zeros_like(w_fc)
+            d_w_proj = torch.zeros_like(w_proj)
+            start = 0
+            for e, end in enumerate(off.tolist()):
+                if end > start:
+                    rows = slice(start, end)
+                    t_e = tok[rows]
+                    d_w_fc[e] = d_h[rows].t() @ x[t_e]
+                    d_w_proj[e] = dy[t_e].t() @ act_g[rows]
+                start = end
         return dx, d_w_fc, d_w_proj, d_gates.to(gates.dtype), None, None, None

@@ -1,0 +1,439 @@
+// Per-expert weight gradients of the scattered-MoE layer on gfx950 matrix cores:
+//
+//   dW[e][m][n] = sum over the rows r of expert e (expert-sorted order) of  A[ai(r)][m] * B[bi(r)][n]
+//
+// i.e. one "X^T dY" product per expert, contracted over that expert's rows.  The reference gets it from the
+// backward of the external scattered_experts op (lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:91-101);
+// its two uses are d c_fc[e] = d_h[rows_e]^T x[token(rows_e)] and d c_proj[e] = dy[token(rows_e)]^T act[rows_e].
+//
+// Design
+//   * Both operands are stored with the contraction index (the row) as the slow dimension, the opposite of what
+//     the matrix instruction wants (8 consecutive contraction values per lane).  The tiles are staged in LDS as
+//     they lie in HBM -- [row][256 columns] -- and the fragments are read with ds_read_b64_tr_b16, which transposes
+//     4 rows x 16 columns across a group of 16 lanes: lane i of the group supplies the address of (row i / 4,
+//     columns 4 * (i % 4) ..) and receives column i of the four rows.  Two such reads make one 16x16x32 operand.
+//     The 32-byte column groups of a row are XOR-swizzled with the row number so that the 16 rows x 32 bytes of
+//     one read spread over the banks.
+//   * An expert's rows are cut into groups of `chunk` rows; a work item is one 256 x 256 output tile of one
+//     group.  Items are dealt so that the 32 workgroups of an XCD work on the tiles of the same few groups at
+//     the same time: the group's rows are then fetched from HBM once per XCD and shared through its L2.
+//     Every item writes an fp32 partial tile; a second kernel sums the partials of an expert in group order
+//     and rounds once (deterministic, and experts without rows get zeros).
+//   * HBM -> LDS by DMA (no registers), a ring of four 32-row slices with three in flight, and the forward
+//     kernel's ping-pong schedule: the two waves of a SIMD alternate between a memory phase and a matrix phase.
+//     A row's address is a scalar (index loads go through the scalar cache), the lanes add constant offsets.
+#include "common.h"
+
+#include <type_traits>
+
+#define WGRAD_MAX_E 256
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+#define MI_LDS __attribute__((address_space(3)))
+
+template <typename T> struct WgradMfma;
+template <> struct WgradMfma<bf16_t> {
+  static __device__ __forceinline__ f32x4 run(s16x8 a, s16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct WgradMfma<f16_t> {
+  static __device__ __forceinline__ f32x4 run(s16x8 a, s16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+
+struct WgradArgs {
+  const void* a;                  // (rows_a, M)
+  const void* b;                  // (rows_b, N)
+  const int32_t* a_idx;           // (L,) row of `a` for sorted row r, or null: r itself
+  const int32_t* b_idx;           // same for `b`
+  const int32_t* expert_offsets;  // (E,) inclusive ends of the experts' row ranges
+  float* partial;                 // [group][M][N]
+  int L, M, N, E, chunk, m_tiles, n_tiles;
+};
+
+__device__ __forceinline__ constexpr int wgrad_waitcnt(int vm, int lgkm) {
+  // gfx9 encoding: vmcnt = {imm[15:14], imm[3:0]}, expcnt = imm[6:4] (7 = no wait), lgkmcnt = imm[11:8]
+  return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 15) << 8);
+}
+
+// etab[2e] = groups of experts 0..e, etab[2e+1] = offsets[e]; returns nothing, all threads must call
+__device__ __forceinline__ void wgrad_build_table(const int32_t* __restrict__ offsets, int E, int chunk, int* etab, int lane,
+                                                  int wave) {
+  if (wave == 0) {
+    int carry = 0;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      const int e = e0 + lane;
+      const int end = e < E ? offsets[e] : 0;
+      const int prev = (e < E && e > 0) ? offsets[e - 1] : 0;
+      int incl = e < E ? (end - prev + chunk - 1) / chunk : 0;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        int v = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += v;
+      }
+      incl += carry;
+      if (e < E) {
+        etab[2 * e] = incl;
+        etab[2 * e + 1] = end;
+      }
+      carry = __shfl(incl, 63, 64);
+    }
+  }
+  __syncthreads();
+}
+
+// Two rows of a tile (512 bytes each) into 1 KiB of LDS starting at `lds_addr`: lanes 0-31 fetch 16 bytes each
+// from base + row_lo + off, lanes 32-63 from base + row_hi + off (32-bit byte offsets); lane l lands at
+// lds_addr + 16 l.  The row offsets are scalars (a gathered operand has an unrelated address per row) and the
+// lane offsets never change; their per-lane sum lives in a register that only this statement names.  Written as
+// assembly for the same reason as in the forward kernel: the compiler would order every later LDS read behind the
+// builtin form of this instruction with vmcnt(0).
+__device__ __forceinline__ void wgrad_dma_row_pair(const void* base, uint32_t row_lo, uint32_t row_hi, uint32_t off,
+                                                   uint64_t upper_half, uint32_t lds_addr) {
+  uint32_t tmp;
+  uint64_t saved;
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_mov_b64 %1, exec\n\t"
+      "v_add_u32 %0, %4, %3\n\t"
+      "s_mov_b64 exec, %7\n\t"
+      "v_add_u32 %0, %5, %3\n\t"
+      "s_mov_b64 exec, %1\n\t"
+      "global_load_lds_dwordx4 %0, %6"
+      : "=&v"(tmp), "=&s"(saved)
+      : "s"(lds_addr), "v"(off), "s"(row_lo), "s"(row_hi), "s"(base), "s"(upper_half)
+      : "memory", "m0");
+}
+
+template <typename T>
+__global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
+  constexpr int BK = 32, TILE = 256;
+  constexpr int OP_BYTES = BK * TILE * 2;  // one operand's 32 rows x 256 columns
+  constexpr int STAGE_BYTES = 2 * OP_BYTES;
+  constexpr int NSTAGE = 4, AHEAD = 3;
+  constexpr int NLD = 4;                   // DMA instructions per wave and slice (4 row pairs)
+  typedef const __attribute__((address_space(4))) int32_t* const_idx_t;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  int* etab = reinterpret_cast<int*>(smem_raw + NSTAGE * STAGE_BYTES);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 3, wn = wave >> 2;
+
+  wgrad_build_table(a.expert_offsets, a.E, a.chunk, etab, lane, wave);
+  const int total_groups = etab[2 * (a.E - 1)];
+  const int tiles = a.m_tiles * a.n_tiles;
+  const int xcd = blockIdx.x & 7, slot0 = blockIdx.x >> 3, nslot = gridDim.x >> 3;
+
+  // An expert with n rows has ceil(n / chunk) groups of equal size (a multiple of 32 rows, the last one shorter).
+  auto group_rows = [&](int n, int groups) { return ((n + groups - 1) / groups + 31) & ~31; };
+  // first group that starts at or after sorted row `b` (wave-uniform)
+  auto group_at = [&](int b) -> int {
+    int res = total_groups;
+    for (int e0 = 0; e0 < a.E; e0 += 64) {
+      const int e = e0 + lane;
+      const int end = e < a.E ? etab[2 * e + 1] : 0x7fffffff;
+      const uint64_t hit = __ballot(end > b);
+      if (hit) {
+        const int ex = e0 + __ffsll((long long)hit) - 1;
+        if (ex < a.E) {
+          const int first = ex > 0 ? etab[2 * (ex - 1)] : 0;
+          const int prev = ex > 0 ? etab[2 * (ex - 1) + 1] : 0;
+          const int groups = etab[2 * ex] - first;
+          const int rows = group_rows(etab[2 * ex + 1] - prev, groups);
+          const int gi = (b - prev + rows - 1) / rows;
+          res = first + (gi < groups ? gi : groups);
+        }
+        break;
+      }
+    }
+    return __builtin_amdgcn_readfirstlane(res);
+  };
+  // every XCD takes the groups that start in its eighth of the sorted rows: equal work up to one group
+  const int gbeg = group_at((int)((long)a.L * xcd >> 3));
+  const int gend = xcd == 7 ? total_groups : group_at((int)((long)a.L * (xcd + 1) >> 3));
+  const int items_x = (gend - gbeg) * tiles;
+
+  // ---- loader role: waves 0-3 stage operand A, waves 4-7 operand B; each wave rows 8 wq .. 8 wq + 7 of a slice --
+  const bool load_b = wave >= 4;
+  const int wq = wave & 3;
+  const unsigned char* src = static_cast<const unsigned char*>(load_b ? a.b : a.a);
+  const const_idx_t idx = reinterpret_cast<const_idx_t>(reinterpret_cast<uintptr_t>(load_b ? a.b_idx : a.a_idx));
+  const bool gathered = idx != nullptr;
+  const int ld = load_b ? a.N : a.M;  // columns of the operand
+  const uint32_t ldbytes32 = (uint32_t)ld * (uint32_t)sizeof(T);  // operands stay below 4 GiB (checked on the host)
+  // LDS position lane % 32 of row `krow` holds the logical 16-byte piece whose 32-byte group is
+  // (position / 2) ^ f(krow), f(krow) = (krow & 3) | (((krow >> 3) & 3) << 2); row pair p of the wave is
+  // krow = 8 wq + 2 p + lane / 32, so f only depends on the parity of p
+  int lcol[2];  // first column (element) of the lane's piece, for even / odd row pairs
+#pragma unroll
+  for (int par = 0; par < 2; ++par) {
+    const int f = ((2 * par + (lane >> 5)) & 3) | (wq << 2);
+    lcol[par] = (((((lane & 31) >> 1) ^ f) & 15) << 4) + (lane & 1) * 8;
+  }
+  const uint32_t lds0 = (uint32_t)(size_t)(MI_LDS void*)smem_raw;
+  const uint32_t wave_lds = lds0 + (load_b ? OP_BYTES : 0) + 8 * wq * (TILE * 2);
+
+  // ---- fragment read addresses (per lane): row 8q + 4h + i/4, column group F ^ f(row), piece i % 4 ----------
+  const int fi = lane & 15, fq = lane >> 4;
+  const int fl = (fi >> 2) | (fq << 2);
+  const uint32_t frag_base = (8 * fq + (fi >> 2)) * (TILE * 2) + (fl << 5) + (fi & 3) * 8;
+
+  for (int item = slot0; item < items_x; item += nslot) {
+    const int grp = gbeg + item / tiles;
+    const int tile = item % tiles;
+    const int mt = tile % a.m_tiles, nt = tile / a.m_tiles;
+
+    // group -> expert and its row range (wave-uniform)
+    int r0 = 0, r1 = 1;
+    for (int e0 = 0; e0 < a.E; e0 += 64) {
+      const int e = e0 + lane;
+      const int incl = e < a.E ? etab[2 * e] : 0x7fffffff;
+      const uint64_t hit = __ballot(incl > grp);
+      if (hit) {
+        const int ex = e0 + __ffsll((long long)hit) - 1;
+        const int first = ex > 0 ? etab[2 * (ex - 1)] : 0;
+        const int prev = ex > 0 ? etab[2 * (ex - 1) + 1] : 0;
+        const int rows = group_rows(etab[2 * ex + 1] - prev, etab[2 * ex] - first);
+        r0 = prev + (grp - first) * rows;
+        r1 = etab[2 * ex + 1];
+        if (r1 > r0 + rows) r1 = r0 + rows;
+        break;
+      }
+    }
+    r0 = __builtin_amdgcn_readfirstlane(r0);
+    r1 = __builtin_amdgcn_readfirstlane(r1);
+    const int nk = (r1 - r0 + BK - 1) / BK;
+
+    // lane offsets of this tile; columns past the operand's width re-read the tile's first piece (their
+    // products only reach output rows / columns that are never stored)
+    const int col0 = (load_b ? nt : mt) * TILE;
+    uint32_t loff[2];
+#pragma unroll
+    for (int par = 0; par < 2; ++par) loff[par] = (uint32_t)((col0 + lcol[par] < ld ? lcol[par] : 0) * sizeof(T));
+    const unsigned char* tile_src = src + (size_t)col0 * sizeof(T);
+
+    // rows of slice `slice` this wave fetches: sorted rows r0 + 32 slice + 8 wq + [0, 8), clamped into the group
+    // (rows past its end are fetched again from its last row and masked out of the last slice's fragments)
+    auto load_idx = [&](int slice, int (&rw)[8]) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        int r = r0 + slice * BK + 8 * wq + i;
+        if (r > r1 - 1) r = r1 - 1;
+        rw[i] = gathered ? idx[r] : r;
+      }
+    };
+    auto dma_slice = [&](const int (&rw)[8], int stage) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p)
+        wgrad_dma_row_pair(tile_src, (uint32_t)rw[2 * p] * ldbytes32, (uint32_t)rw[2 * p + 1] * ldbytes32, loff[p & 1],
+                           0xffffffff00000000ull, wave_lds + stage * STAGE_BYTES + 2 * p * (TILE * 2));
+    };
+
+    f32x4 acc[4][8];
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < 8; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    s16x8 af[4], bf[8];
+    auto read_frag = [&](int stage, int opoff, int F) -> s16x8 {
+      const uint32_t addr = lds0 + stage * STAGE_BYTES + opoff + (frag_base ^ ((uint32_t)F << 5));
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MI_LDS s16x4*)(size_t)addr);
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MI_LDS s16x4*)(size_t)(addr + 4 * TILE * 2));
+      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    auto read_frags = [&](int stage) {
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) af[mb] = read_frag(stage, 0, 4 * wm + mb);
+#pragma unroll
+      for (int nb = 0; nb < 8; ++nb) bf[nb] = read_frag(stage, OP_BYTES, 8 * wn + nb);
+    };
+    auto multiply = [&]() {
+#pragma unroll
+      for (int nb = 0; nb < 8; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) acc[mb][nb] = WgradMfma<T>::run(af[mb], bf[nb], acc[mb][nb]);
+    };
+    // the last slice of a group may be short: element j of a fragment is row 8 (lane / 16) + j of the slice
+    const int last_rows = r1 - r0 - (nk - 1) * BK;
+    auto mask_frags = [&]() {
+      uint32_t m[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int k = 8 * fq + 2 * t;
+        m[t] = (k < last_rows ? 0x0000ffffu : 0u) | (k + 1 < last_rows ? 0xffff0000u : 0u);
+      }
+      auto apply = [&](s16x8& v) {
+        u32x4 w = __builtin_bit_cast(u32x4, v);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) w[t] &= m[t];
+        v = __builtin_bit_cast(s16x8, w);
+      };
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) apply(af[mb]);
+#pragma unroll
+      for (int nb = 0; nb < 8; ++nb) apply(bf[nb]);
+    };
+
+    // ---- K loop: the forward kernel's ping-pong schedule.  The waves wn == 0 and wn == 1 (one of each per SIMD)
+    // run the same code one phase apart: while one group issues its 32 matrix instructions out of registers, the
+    // other reads its fragments of the slice and issues its share of the DMA for the slice three ahead.
+    int rw[8];
+    load_idx(0, rw);
+    dma_slice(rw, 0);
+    load_idx(1, rw);
+    dma_slice(rw, 1);
+    load_idx(2, rw);
+    dma_slice(rw, 2);
+    load_idx(3, rw);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(wgrad_waitcnt((AHEAD - 1) * NLD, 0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (wn == 1) __builtin_amdgcn_s_barrier();
+    for (int g = 0; g < nk; ++g) {
+      const int cur = g & (NSTAGE - 1), fill = (g + AHEAD) & (NSTAGE - 1);
+      read_frags(cur);
+      // slices past the group's end are fetched like the others (clamped rows) and never multiplied
+      dma_slice(rw, fill);
+      if (g == nk - 1 && last_rows < BK) mask_frags();
+      asm volatile("" ::: "memory");
+      // own DMA of slice g + 1 has landed (g + 2 and g + 3 stay in flight); fragments are in registers
+      __builtin_amdgcn_s_waitcnt(wgrad_waitcnt((NSTAGE - 2) * NLD, 0));
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      // the row indices of the next DMA come in through the scalar cache while the matrix pipe works
+      load_idx(g + 4, rw);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply();
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (wn == 0) __builtin_amdgcn_s_barrier();
+    // surplus DMA (slices nk .. nk + 2) must land before the next item reuses the ring
+    __builtin_amdgcn_s_waitcnt(wgrad_waitcnt(0, 0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    // ---- fp32 partial tile: register i of block (mb, nb) is row 16 mb + 4 (lane / 16) + i, column 16 nb + lane % 16
+    float* __restrict__ out = a.partial + (size_t)grp * a.M * a.N;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = mt * TILE + wm * 64 + mb * 16 + 4 * fq + i;
+        if (m < a.M) {
+#pragma unroll
+          for (int nb = 0; nb < 8; ++nb) {
+            const int n = nt * TILE + wn * 128 + nb * 16 + fi;
+            if (n < a.N) out[(size_t)m * a.N + n] = acc[mb][nb][i];
+          }
+        }
+      }
+  }
+}
+
+// dW[e] = sum of expert e's partial slabs in group order, rounded once; zeros for an expert without rows
+template <typename T>
+__global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ partial,
+                                                           const int32_t* __restrict__ offsets, T* __restrict__ dw,
+                                                           int E, long mn, int chunk) {
+  const int e = blockIdx.y;
+  int first = 0, prev = 0;
+  for (int i = 0; i < e; ++i) {
+    const int end = offsets[i];
+    first += (end - prev + chunk - 1) / chunk;
+    prev = end;
+  }
+  const int count = (offsets[e] - prev + chunk - 1) / chunk;
+  const long n8 = mn / 8;
+  for (long id = (long)blockIdx.x * 256 + threadIdx.x; id < n8; id += (long)gridDim.x * 256) {
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    for (int g = 0; g < count; ++g) {
+      const float* p = partial + (size_t)(first + g) * mn + id * 8;
+      const f32x4 v0 = *reinterpret_cast<const f32x4*>(p);
+      const f32x4 v1 = *reinterpret_cast<const f32x4*>(p + 4);
+      s0 += v0;
+      s1 += v1;
+    }
+    u32x4 o;
+    o[0] = pack2<T>(s0[0], s0[1]);
+    o[1] = pack2<T>(s0[2], s0[3]);
+    o[2] = pack2<T>(s1[0], s1[1]);
+    o[3] = pack2<T>(s1[2], s1[3]);
+    *reinterpret_cast<u32x4*>(dw + (size_t)e * mn + id * 8) = o;
+  }
+}
+
+// rows per group: enough groups for about four items per CU, between 256 and 8192 rows, a multiple of 32
+static int wgrad_chunk(int L, int M, int N) {
+  const long tiles = (long)mi_ceil_div(M, 256) * mi_ceil_div(N, 256);
+  long groups = (1024 + tiles - 1) / tiles;
+  long chunk = L / (groups > 0 ? groups : 1);
+  if (chunk > 8192) chunk = 8192;
+  if (chunk < 256) chunk = 256;
+  return (int)(chunk / 32 * 32);
+}
+
+static long wgrad_max_groups(int L, int E, int chunk) { return (long)L / chunk + (E < L ? E : L); }
+
+extern "C" size_t mi_moe_grouped_wgrad_workspace_bytes(int L, int E, int M, int N) {
+  if (L < 1 || E < 1 || M < 1 || N < 1) return 0;
+  return (size_t)wgrad_max_groups(L, E, wgrad_chunk(L, M, N)) * (size_t)M * (size_t)N * sizeof(float);
+}
+
+extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const void* b, const int32_t* b_idx,
+                                    const int32_t* expert_offsets, void* dw, void* workspace, size_t workspace_bytes,
+                                    int L, int a_rows, int b_rows, int M, int N, int E, int dtype, mi_moe_stream_t stream) {
+  if (L < 0 || M < 1 || N < 1 || E < 1) return MI_MOE_ESHAPE;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (M % 8 != 0 || N % 8 != 0 || E > WGRAD_MAX_E) return MI_MOE_EUNSUPPORTED;
+  if (a_rows < 0 || b_rows < 0) return MI_MOE_ESHAPE;
+  // rows are addressed with 32-bit byte offsets
+  if ((uint64_t)a_rows * M * 2 >= (1ull << 32) || (uint64_t)b_rows * N * 2 >= (1ull << 32)) return MI_MOE_EUNSUPPORTED;
+  if (!dw || !expert_offsets) return MI_MOE_ENULL;
+  if (L > 0 && (!a || !b)) return MI_MOE_ENULL;
+  if (!mi_aligned(a, 16) || !mi_aligned(b, 16) || !mi_aligned(dw, 16) || !mi_aligned(workspace, 16)) return MI_MOE_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const long mn = (long)M * N;
+  if (L > 0 && (!workspace || workspace_bytes < mi_moe_grouped_wgrad_workspace_bytes(L, E, M, N))) return MI_MOE_EWORKSPACE;
+
+  WgradArgs g;
+  g.a = a; g.b = b; g.a_idx = a_idx; g.b_idx = b_idx; g.expert_offsets = expert_offsets;
+  g.partial = static_cast<float*>(workspace);
+  g.L = L; g.M = M; g.N = N; g.E = E;
+  g.chunk = wgrad_chunk(L, M, N);
+  g.m_tiles = mi_ceil_div(M, 256);
+  g.n_tiles = mi_ceil_div(N, 256);
+  const size_t lds = 4 * 2 * 32 * 256 * 2 + (size_t)E * 8;
+  int dev = 0, cus = 0;
+  hipError_t e;
+  if ((e = hipGetDevice(&dev)) != hipSuccess) return (int)e;
+  if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return (int)e;
+  const long max_items = wgrad_max_groups(L, E, g.chunk) * g.m_tiles * g.n_tiles;
+  long grid = cus < max_items ? cus : max_items;
+  grid = (grid + 7) / 8 * 8;
+  long rblocks = (mn / 8 + 255) / 256;
+  if (rblocks > 4096) rblocks = 4096;
+  if (dtype == MI_MOE_BF16) {
+    auto kern = grouped_wgrad_kernel<bf16_t>;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess)
+      return (int)e;
+    if (L > 0) hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, s, g);
+    hipLaunchKernelGGL((wgrad_reduce_kernel<bf16_t>), dim3((unsigned)rblocks, (unsigned)E), dim3(256), 0, s, g.partial,
+                       expert_offsets, static_cast<bf16_t*>(dw), E, mn, g.chunk);
+  } else {
+    auto kern = grouped_wgrad_kernel<f16_t>;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess)
+      return (int)e;
+    if (L > 0) hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, s, g);
+    hipLaunchKernelGGL((wgrad_reduce_kernel<f16_t>), dim3((unsigned)rblocks, (unsigned)E), dim3(256), 0, s, g.partial,
+                       expert_offsets, static_cast<f16_t*>(dw), E, mn, g.chunk);
+  }
+  return mi_launch_status();
+}

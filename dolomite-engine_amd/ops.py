@@ -318,6 +318,48 @@ def combine_grad_gates(o: torch.Tensor, dy: torch.Tensor, k: int) -> torch.Tenso
     return d_gates
 
 
+def grouped_wgrad_supported(a: torch.Tensor, b: torch.Tensor, num_experts: int) -> bool:
+    return (a.dtype in (torch.float16, torch.bfloat16) and a.shape[1] % 8 == 0 and b.shape[1] % 8 == 0
+            and num_experts <= 256 and a.numel() * 2 < 2 ** 32 and b.numel() * 2 < 2 ** 32)
+
+
+def grouped_wgrad(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor,
+                  a_idx: torch.Tensor | None = None, b_idx: torch.Tensor | None = None) -> torch.Tensor:
+    """dw[e] = sum over the sorted rows r of expert e of outer(a[ai(r)], b[bi(r)]), (E, M, N).
+
+    ``a`` (rows_a, M) and ``b`` (rows_b, N) are 16-bit; ``a_idx`` / ``b_idx`` (L,) int32 map a sorted row to a
+    row of the operand (``None``: the operand is already in sorted order and has L rows).  The per-expert
+    weight gradient of the backward of ``scattered_experts`` (moe.py:91-101)."""
+    _dev(a, b, expert_offsets, a_idx, b_idx)
+    _no_grad(a, b)
+    a = a.contiguous()
+    b = b.contiguous()
+    E = expert_offsets.shape[0]
+    M, N = a.shape[1], b.shape[1]
+    if a.dtype != b.dtype:
+        raise ValueError("a and b must have the same dtype")
+    L = None
+    for t, i in ((a, a_idx), (b, b_idx)):
+        n = t.shape[0] if i is None else i.shape[0]
+        if i is not None and (i.dtype != torch.int32 or i.dim() != 1):
+            raise ValueError("index arrays must be 1-D int32")
+        if L is not None and n != L:
+            raise ValueError("a and b disagree on the number of sorted rows")
+        L = n
+    a_idx = None if a_idx is None else a_idx.contiguous()
+    b_idx = None if b_idx is None else b_idx.contiguous()
+    expert_offsets = expert_offsets.contiguous()
+    lib = _lib.load()
+    ws_bytes = int(lib.mi_moe_grouped_wgrad_workspace_bytes(L, E, M, N))
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=a.device)
+    dw = torch.empty((E, M, N), dtype=a.dtype, device=a.device)
+    with _stage("grouped_wgrad"):
+        check(lib.mi_moe_grouped_wgrad(_ptr(a), _ptr(a_idx), _ptr(b), _ptr(b_idx), _ptr(expert_offsets), _ptr(dw),
+                                       _ptr(ws), ws_bytes, L, a.shape[0], b.shape[0], M, N, E, _code(a.dtype),
+                                       _stream()))
+    return dw
+
+
 def scattered_experts(inputs: torch.Tensor, expert_weights: torch.Tensor, k: int,
                       sorted_expert_idxs: torch.Tensor, sorted_scattered_idxs: torch.Tensor,
                       expert_offsets: torch.Tensor, gates: torch.Tensor | None = None, grouped_in: bool = False,

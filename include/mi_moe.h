@@ -194,6 +194,22 @@ int mi_moe_combine_grad_gates(const void* o, const void* dy, void* d_gates, int 
                               mi_moe_stream_t stream);
 
 /*
+ * Per-expert weight gradients (the "X^T dY" of the backward of scattered_experts, moe.py:91-101):
+ *     dw[e, m, n] = sum over sorted rows r of expert e of  a[ai(r), m] * b[bi(r), n]
+ * with ai(r) = a_idx[r] (or r if a_idx is NULL), same for b.  a (rows_a, M), b (rows_b, N), dw (E, M, N) of
+ * `dtype` (F16 / BF16), fp32 accumulation, one rounding.  Deterministic: an expert's rows are summed in a fixed
+ * order (partial sums per group of rows in the workspace, then added up in group order); experts without rows
+ * get zeros.  M % 8 == 0, N % 8 == 0, E <= 256 and both operands below 4 GiB (a_rows, b_rows: their row counts),
+ * else MI_MOE_EUNSUPPORTED.  Index values are not checked.
+ * Uses: d c_fc[e] = d_h[rows]^T x[token(rows)] (a = d_h in sorted order, b = x gathered), and
+ *       d c_proj[e] = dy[token(rows)]^T act[rows] (a = dy gathered, b = act in sorted order).
+ */
+size_t mi_moe_grouped_wgrad_workspace_bytes(int L, int E, int M, int N);
+int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const void* b, const int32_t* b_idx,
+                         const int32_t* expert_offsets, void* dw, void* workspace, size_t workspace_bytes,
+                         int L, int a_rows, int b_rows, int M, int N, int E, int dtype, mi_moe_stream_t stream);
+
+/*
  * Decode-shape variants with fp8 (OCP e4m3fn) expert weights and one fp32 scale per output channel.
  * No counterpart in the reference (its fp8 support wraps nn.Linear only, lm_engine/fp8.py:63-73);
  * semantics = dequantise (w * scale[:, None]) then the two calls above.

@@ -70,3 +70,79 @@ def test_combine_grad_gates(device, dtype, T, k, H):
     eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
     # an fp32 dot product of H terms rounded once; the absolute term covers cancellation
     torch.testing.assert_close(got.cpu().float(), gates.grad, rtol=2 * eps, atol=1e-4 * H ** 0.5)
+
+
+def _wgrad_reference(a, b, offsets, a_idx, b_idx):
+    """fp64 loop over experts: the definition, with plain matrix products."""
+    E = offsets.shape[0]
+    out = torch.zeros(E, a.shape[1], b.shape[1], dtype=torch.float64)
+    start = 0
+    for e, end in enumerate(offsets.tolist()):
+        if end > start:
+            rows = torch.arange(start, end)
+            ar = a[a_idx[rows].long()] if a_idx is not None else a[rows]
+            br = b[b_idx[rows].long()] if b_idx is not None else b[rows]
+            out[e] = ar.double().t() @ br.double()
+        start = end
+    return out
+
+
+WGRAD_CASES = [
+    # L, E, M, N, rows_other (rows of the gathered operand)
+    (1, 1, 8, 8, 1),
+    (33, 3, 16, 24, 9),
+    (700, 8, 256, 256, 350),
+    (1500, 5, 264, 520, 200),      # ragged column tiles on both operands
+    (5000, 40, 512, 128, 625),     # many experts, several row groups per expert
+    (2100, 130, 64, 72, 300),      # more experts than one ballot covers
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("L,E,M,N,rows_other", WGRAD_CASES)
+@pytest.mark.parametrize("gather", ["a", "b", "none", "both"])
+def test_grouped_wgrad(device, dtype, L, E, M, N, rows_other, gather):
+    g = torch.Generator().manual_seed(L * 7 + E)
+    # skewed expert sizes with empty experts in between
+    w = torch.rand(E, generator=g).pow(3)
+    w[torch.rand(E, generator=g) < 0.25] = 0
+    if w.sum() == 0:
+        w[0] = 1
+    counts = torch.distributions.Multinomial(L, w / w.sum()).sample().long() if L > 1 else torch.tensor([L] + [0] * (E - 1))
+    offsets = counts.cumsum(0).to(torch.int32)
+    assert int(offsets[-1]) == L
+    ga, gb = gather in ("a", "both"), gather in ("b", "both")
+    a = torch.randn(rows_other if ga else L, M, generator=g).to(dtype)
+    b = torch.randn(rows_other if gb else L, N, generator=g).to(dtype)
+    a_idx = torch.randint(0, rows_other, (L,), generator=g, dtype=torch.int32) if ga else None
+    b_idx = torch.randint(0, rows_other, (L,), generator=g, dtype=torch.int32) if gb else None
+
+    got = _ops().grouped_wgrad(a.to(device), b.to(device), offsets.to(device),
+                               None if a_idx is None else a_idx.to(device), None if b_idx is None else b_idx.to(device))
+    assert got.dtype == dtype and tuple(got.shape) == (E, M, N)
+    ref = _wgrad_reference(a, b, offsets, a_idx, b_idx)
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    # fp32 accumulation of up to L products of unit-variance terms, one rounding to the dtype
+    torch.testing.assert_close(got.cpu().double(), ref, rtol=2 * eps, atol=2e-5 * max(1.0, counts.max().item()) ** 0.5 + 1e-6)
+    # experts without rows get exact zeros
+    for e in (counts == 0).nonzero().flatten().tolist():
+        assert not got[e].any()
+
+
+def test_grouped_wgrad_is_deterministic(device):
+    g = torch.Generator().manual_seed(5)
+    L, E, M, N = 9000, 6, 256, 512
+    a = torch.randn(L, M, generator=g).to(torch.bfloat16).to(device)
+    b = torch.randn(L, N, generator=g).to(torch.bfloat16).to(device)
+    offsets = torch.tensor([4000, 4000, 4100, 8000, 8990, 9000], dtype=torch.int32, device=device)
+    first = _ops().grouped_wgrad(a, b, offsets)
+    for _ in range(3):
+        assert torch.equal(_ops().grouped_wgrad(a, b, offsets), first)
+
+
+def test_grouped_wgrad_no_rows(device):
+    ops = _ops()
+    a = torch.empty(0, 16, dtype=torch.bfloat16, device=device)
+    b = torch.empty(0, 8, dtype=torch.bfloat16, device=device)
+    out = ops.grouped_wgrad(a, b, torch.zeros(4, dtype=torch.int32, device=device))
+    assert tuple(out.shape) == (4, 16, 8) and not out.any()
