@@ -8,8 +8,9 @@ gradients (fp32 and odd shapes fall back to one library GEMM per expert).  The r
 (lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:91-101); this module is the counterpart for the
 gradient, built on this package's forward kernels.
 
-Memory kept for the backward: x, the gates, the routing indices and the (L, I) activation; the (L, 2I)
-pre-activation and the (L, H) expert outputs are recomputed.
+Memory kept for the backward: x, the gates and the routing indices; the (L, 2I) pre-activation is recomputed,
+the (L, I) activation follows from it, and the (L, H) expert outputs are never needed (the gradient of a router
+weight, <dy[t], w_proj[e] a>, is taken as <w_proj[e]^T dy[t], a>).
 """
 
 from __future__ import annotations
@@ -27,58 +28,55 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
         act = ops.up_swiglu(x, w_fc, k, sorted_scattered, expert_offsets)
         o = ops.scattered_gemm(act, w_proj, 1, sorted_scattered, expert_offsets, True, False)
         y = ops.combine(o, gates)
-        ctx.save_for_backward(x, w_fc, w_proj, gates, sorted_scattered, expert_offsets, act)
+        ctx.save_for_backward(x, w_fc, w_proj, gates, sorted_scattered, expert_offsets)
         ctx.k = k
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        x, w_fc, w_proj, gates, ss, off, act = ctx.saved_tensors
+        x, w_fc, w_proj, gates, ss, off = ctx.saved_tensors
         k = ctx.k
         T, H = x.shape
         E, I2, _ = w_fc.shape
         I = I2 // 2
         dy = dy.contiguous()
-        ssl = ss.long()
-        tok = ssl // k                                # token of every sorted row
-        g_sorted = gates.reshape(-1)[ssl]             # gate of every sorted row
+        half = x.dtype in (torch.float16, torch.bfloat16) and I % 8 == 0
 
-        half = x.dtype in (torch.float16, torch.bfloat16)
-
-        # gradient w.r.t. the gates: <dy[t], o[t, j]>, o recomputed from the kept activation
-        o = ops.scattered_gemm(act, w_proj, 1, ss, off, True, False)
-        if half and H % 8 == 0:
-            d_gates = ops.combine_grad_gates(o, dy, k)
-        else:
-            d_gates = torch.bmm(o.view(T, k, H), dy.unsqueeze(-1)).squeeze(-1)
-        del o
-
-        # gradient w.r.t. the SwiGLU output, in grouped order: dy[t_i] @ w_proj[e_i]; the gate g_i of the row
-        # is applied together with the SwiGLU backward on the recomputed pre-activation
+        # gradient w.r.t. the SwiGLU output a, in sorted order and before the router weight: dy[t_i] @ w_proj[e_i]
         d_act = ops.scattered_gemm(dy, w_proj.transpose(1, 2).contiguous(), k, ss, off, False, True)
+        # pre-activation recomputed; one pass then gives d_h (with the router weight g_i of the row applied),
+        # g_i * a_i for the down-projection's weight gradient, and the gradient of the router weights,
+        # <dy[t], w_proj[e] a_i> = <d_act_i, a_i>
         h = ops.scattered_gemm(x, w_fc, k, ss, off, False, True)
-        if half and I % 8 == 0:
-            d_h = ops.swiglu_backward(h, d_act, g_sorted)
+        if half:
+            d_h, act_g, d_gates = ops.swiglu_backward(h, d_act, gates, ss, want_act=True, want_gate_grad=True)
         else:
-            up, gate = h[:, :I].float(), h[:, I:].float()
+            ssl = ss.long()
+            g_sorted = gates.reshape(-1)[ssl].float().unsqueeze(-1)
+            up, gate, da = h[:, :I].float(), h[:, I:].float(), d_act.float()
             sig = torch.sigmoid(gate)
-            da = d_act.float() * g_sorted.float().unsqueeze(-1)
+            a = up * gate * sig
+            d_gates = torch.empty(T * k, dtype=torch.float32, device=x.device)
+            d_gates[ssl] = (da * a).sum(dim=1)
+            d_gates = d_gates.view(T, k).to(gates.dtype)
+            da = da * g_sorted
             d_h = torch.cat([da * gate * sig, da * up * sig * (1.0 + gate * (1.0 - sig))], dim=1).to(x.dtype)
-            del up, gate, sig, da
+            act_g = (a * g_sorted).to(x.dtype)
+            del up, gate, sig, da, a
         del h, d_act
 
         # gradient w.r.t. x: every slot's contribution in flat-slot order, then the k slots of a token summed
         dx_slots = ops.scattered_gemm(d_h, w_fc.transpose(1, 2).contiguous(), 1, ss, off, True, False)
-        dx = dx_slots.view(T, k, H).sum(dim=1)
+        dx = ops.combine(dx_slots, torch.ones_like(gates))
         del dx_slots
 
         # weight gradients: per expert X^T dY over that expert's rows
-        act_g = act * g_sorted.unsqueeze(-1)          # (g dy)^T a == dy^T (g a), and a is the narrower of the two
+        tok32 = torch.div(ss, k, rounding_mode="floor").to(torch.int32)
         if half and ops.grouped_wgrad_supported(d_h, x, E):
-            tok32 = tok.to(torch.int32)
             d_w_fc = ops.grouped_wgrad(d_h, x, off, None, tok32)
             d_w_proj = ops.grouped_wgrad(dy, act_g, off, tok32, None)
         else:
+            tok = tok32.long()
             d_w_fc = torch.zeros_like(w_fc)
             d_w_proj = torch.zeros_like(w_proj)
             start = 0
@@ -89,4 +87,4 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
                     d_w_fc[e] = d_h[rows].t() @ x[t_e]
                     d_w_proj[e] = dy[t_e].t() @ act_g[rows]
                 start = end
-        return dx, d_w_fc, d_w_proj, d_gates.to(gates.dtype), None, None, None
+        return dx, d_w_fc, d_w_proj, d_gates, None, None, None

@@ -2,47 +2,65 @@
 //
 //   swiglu_backward:     a = up * silu(gate)  =>  d_up = d_a * silu(gate),
 //                        d_gate = d_a * up * sigmoid(gate) * (1 + gate * (1 - sigmoid(gate)))
-//                        with an optional per-row factor on d_a (the gate weight of the row's slot);
-//                        the forward is GLUActivation with SiLU, lm_engine/hf_models/modeling_utils/activations/glu.py:42-43.
+//                        (the forward is GLUActivation with SiLU,
+//                        lm_engine/hf_models/modeling_utils/activations/glu.py:42-43).  With the router weight g
+//                        of the row's slot, d_a is taken as g * d_act, and the same pass can emit g * a (the
+//                        operand of the down-projection's weight gradient) and <d_act, a>, which is the gradient
+//                        of the slot's router weight: <dy[t], W a> = <W^T dy[t], a>.
 //   combine_grad_gates:  y[t] = sum_j g[t, j] * o[t*k + j]  =>  d_g[t, j] = <dy[t], o[t*k + j]>
 //                        (the gates contraction of moe.py:282-290).
 // fp32 arithmetic, one rounding to the model dtype.
 #include "common.h"
 
+// one wave per sorted row: the lanes stride over the row in 16-byte chunks
 template <typename T>
 __global__ __launch_bounds__(256) void swiglu_backward_kernel(const T* __restrict__ h, const T* __restrict__ d_act,
-                                                              const T* __restrict__ row_scale, T* __restrict__ d_h,
-                                                              int L, int I) {
-  // a thread owns 8 consecutive columns (16 bytes of a 16-bit type) of one row
+                                                              const T* __restrict__ gates,
+                                                              const int32_t* __restrict__ sorted_scattered,
+                                                              T* __restrict__ d_h, T* __restrict__ act_g,
+                                                              T* __restrict__ d_gates, int L, int I) {
+  const int lane = threadIdx.x & 63;
   const int cpr = I / 8;
-  const long total = (long)L * cpr;
-  for (long id = (long)blockIdx.x * 256 + threadIdx.x; id < total; id += (long)gridDim.x * 256) {
-    const int row = (int)(id / cpr);
-    const int c = (int)(id - (long)row * cpr) * 8;
+  for (int row = blockIdx.x * 4 + (threadIdx.x >> 6); row < L; row += gridDim.x * 4) {
+    const int slot = sorted_scattered != nullptr ? sorted_scattered[row] : row;
+    const float g = gates != nullptr ? Elt<T>::load(gates + slot) : 1.0f;
     const T* hr = h + (size_t)row * 2 * I;
-    const u32x4 vu = *reinterpret_cast<const u32x4*>(hr + c);
-    const u32x4 vg = *reinterpret_cast<const u32x4*>(hr + I + c);
-    const u32x4 vd = *reinterpret_cast<const u32x4*>(d_act + (size_t)row * I + c);
-    const float s = row_scale != nullptr ? Elt<T>::load(row_scale + row) : 1.0f;
-    u32x4 ou, og;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float du[2], dg[2];
-#pragma unroll
-      for (int p = 0; p < 2; ++p) {
-        const float up = p ? unpack_hi<T>(vu[i]) : unpack_lo<T>(vu[i]);
-        const float gt = p ? unpack_hi<T>(vg[i]) : unpack_lo<T>(vg[i]);
-        const float da = (p ? unpack_hi<T>(vd[i]) : unpack_lo<T>(vd[i])) * s;
-        const float sig = 1.0f / (1.0f + __expf(-gt));
-        du[p] = da * gt * sig;
-        dg[p] = da * up * sig * (1.0f + gt * (1.0f - sig));
-      }
-      ou[i] = pack2<T>(du[0], du[1]);
-      og[i] = pack2<T>(dg[0], dg[1]);
-    }
     T* dr = d_h + (size_t)row * 2 * I;
-    *reinterpret_cast<u32x4*>(dr + c) = ou;
-    *reinterpret_cast<u32x4*>(dr + I + c) = og;
+    float dot = 0.f;
+    for (int c = lane; c < cpr; c += 64) {
+      const u32x4 vu = *reinterpret_cast<const u32x4*>(hr + c * 8);
+      const u32x4 vg = *reinterpret_cast<const u32x4*>(hr + I + c * 8);
+      const u32x4 vd = *reinterpret_cast<const u32x4*>(d_act + (size_t)row * I + c * 8);
+      u32x4 ou, og, oa;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float du[2], dg[2], ag[2];
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          const float up = p ? unpack_hi<T>(vu[i]) : unpack_lo<T>(vu[i]);
+          const float gt = p ? unpack_hi<T>(vg[i]) : unpack_lo<T>(vg[i]);
+          const float da = p ? unpack_hi<T>(vd[i]) : unpack_lo<T>(vd[i]);
+          const float sig = 1.0f / (1.0f + __expf(-gt));
+          const float act = up * gt * sig;
+          dot = fmaf(da, act, dot);
+          const float das = da * g;
+          du[p] = das * gt * sig;
+          dg[p] = das * up * sig * (1.0f + gt * (1.0f - sig));
+          ag[p] = act * g;
+        }
+        ou[i] = pack2<T>(du[0], du[1]);
+        og[i] = pack2<T>(dg[0], dg[1]);
+        oa[i] = pack2<T>(ag[0], ag[1]);
+      }
+      *reinterpret_cast<u32x4*>(dr + c * 8) = ou;
+      *reinterpret_cast<u32x4*>(dr + I + c * 8) = og;
+      if (act_g != nullptr) *reinterpret_cast<u32x4*>(act_g + (size_t)row * I + c * 8) = oa;
+    }
+    if (d_gates != nullptr) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, MI_WAVE);
+      if (lane == 0) Elt<T>::store(d_gates + slot, dot);
+    }
   }
 }
 
@@ -72,25 +90,28 @@ __global__ __launch_bounds__(256) void combine_grad_gates_kernel(const T* __rest
   }
 }
 
-extern "C" int mi_moe_swiglu_backward(const void* h, const void* d_act, const void* row_scale, void* d_h, int L, int I,
-                                      int dtype, mi_moe_stream_t stream) {
+extern "C" int mi_moe_swiglu_backward(const void* h, const void* d_act, const void* gates,
+                                      const int32_t* sorted_scattered, void* d_h, void* act_g, void* d_gates, int L,
+                                      int I, int dtype, mi_moe_stream_t stream) {
   if (L < 0 || I < 1) return MI_MOE_ESHAPE;
   if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
   if (I % 8 != 0) return MI_MOE_EUNSUPPORTED;
   if (L == 0) return MI_MOE_OK;
   if (!h || !d_act || !d_h) return MI_MOE_ENULL;
-  if (!mi_aligned(h, 16) || !mi_aligned(d_act, 16) || !mi_aligned(d_h, 16)) return MI_MOE_EALIGN;
+  if (!mi_aligned(h, 16) || !mi_aligned(d_act, 16) || !mi_aligned(d_h, 16) || !mi_aligned(act_g, 16)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  long blocks = ((long)L * (I / 8) + 255) / 256;
+  long blocks = ((long)L + 3) / 4;
   if (blocks > 256L * 64) blocks = 256L * 64;
   if (dtype == MI_MOE_BF16)
     hipLaunchKernelGGL((swiglu_backward_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s,
                        static_cast<const bf16_t*>(h), static_cast<const bf16_t*>(d_act),
-                       static_cast<const bf16_t*>(row_scale), static_cast<bf16_t*>(d_h), L, I);
+                       static_cast<const bf16_t*>(gates), sorted_scattered, static_cast<bf16_t*>(d_h),
+                       static_cast<bf16_t*>(act_g), static_cast<bf16_t*>(d_gates), L, I);
   else
     hipLaunchKernelGGL((swiglu_backward_kernel<f16_t>), dim3((unsigned)blocks), dim3(256), 0, s,
-                       static_cast<const f16_t*>(h), static_cast<const f16_t*>(d_act),
-                       static_cast<const f16_t*>(row_scale), static_cast<f16_t*>(d_h), L, I);
+                       static_cast<const f16_t*>(h), static_cast<const f16_t*>(d_act), static_cast<const f16_t*>(gates),
+                       sorted_scattered, static_cast<f16_t*>(d_h), static_cast<f16_t*>(act_g),
+                       static_cast<f16_t*>(d_gates), L, I);
   return mi_launch_status();
 }
 

@@ -281,25 +281,40 @@ def combine(o: torch.Tensor, gates: torch.Tensor, shared: torch.Tensor | None = 
     return y
 
 
-def swiglu_backward(h: torch.Tensor, d_act: torch.Tensor, row_scale: torch.Tensor | None = None) -> torch.Tensor:
-    """Gradient of ``a = h[:, :I] * silu(h[:, I:])`` (activations/glu.py:42-43) w.r.t. ``h`` given ``d_act``
-    (L, I); ``row_scale`` (L,) multiplies ``d_act`` per row first.  16-bit dtypes."""
-    _dev(h, d_act, row_scale)
+def swiglu_backward(h: torch.Tensor, d_act: torch.Tensor, gates: torch.Tensor | None = None,
+                    sorted_scattered_idxs: torch.Tensor | None = None, want_act: bool = False,
+                    want_gate_grad: bool = False):
+    """Backward of ``a = h[:, :I] * silu(h[:, I:])`` (activations/glu.py:42-43) over the sorted rows.
+
+    ``d_act`` (L, I) is the gradient w.r.t. ``a`` before the router weight; row i is scaled by
+    ``g_i = gates.flatten()[sorted_scattered_idxs[i]]`` (1 without ``gates``).  Returns ``(d_h, act_g, d_gates)``:
+    ``d_h`` (L, 2I); ``act_g = g * a`` (L, I) if ``want_act``; ``d_gates`` in the shape of ``gates`` with
+    ``<d_act[i], a[i]>`` at the slot of row i if ``want_gate_grad``.  16-bit dtypes."""
+    _dev(h, d_act, gates, sorted_scattered_idxs)
     _no_grad(h, d_act)
     h = h.contiguous()
     d_act = d_act.contiguous()
     L, I = d_act.shape
     if tuple(h.shape) != (L, 2 * I) or h.dtype != d_act.dtype:
         raise ValueError("h must be (L, 2I) and d_act (L, I) of the same dtype")
-    if row_scale is not None:
-        row_scale = row_scale.contiguous()
-        if tuple(row_scale.shape) != (L,) or row_scale.dtype != h.dtype:
-            raise ValueError("row_scale must be (L,) in the dtype of h")
+    if gates is not None:
+        gates = gates.contiguous()
+        if gates.numel() != L or gates.dtype != h.dtype:
+            raise ValueError("gates must have one entry per row in the dtype of h")
+    if sorted_scattered_idxs is not None:
+        sorted_scattered_idxs = sorted_scattered_idxs.contiguous()
+        if tuple(sorted_scattered_idxs.shape) != (L,) or sorted_scattered_idxs.dtype != torch.int32:
+            raise ValueError("sorted_scattered_idxs must be (L,) int32")
+    if want_gate_grad and gates is None:
+        raise ValueError("want_gate_grad needs gates")
     d_h = torch.empty_like(h)
+    act_g = torch.empty_like(d_act) if want_act else None
+    d_gates = torch.empty_like(gates) if want_gate_grad else None
     with _stage("swiglu_backward"):
-        check(_lib.load().mi_moe_swiglu_backward(_ptr(h), _ptr(d_act), _ptr(row_scale), _ptr(d_h), L, I,
-                                                 _code(h.dtype), _stream()))
-    return d_h
+        check(_lib.load().mi_moe_swiglu_backward(_ptr(h), _ptr(d_act), _ptr(gates), _ptr(sorted_scattered_idxs),
+                                                 _ptr(d_h), _ptr(act_g), _ptr(d_gates), L, I, _code(h.dtype),
+                                                 _stream()))
+    return d_h, act_g, d_gates
 
 
 def combine_grad_gates(o: torch.Tensor, dy: torch.Tensor, k: int) -> torch.Tensor:

@@ -183,12 +183,17 @@ int mi_moe_combine_block_tail(const void* o, const void* gates, const void* shar
  * gradients from the autograd function of the external scattermoe package (moe.py:91-101); these two are
  * the parts of that backward that are neither a grouped GEMM nor a library GEMM.  F16 / BF16 only.
  *
- * mi_moe_swiglu_backward: h (L, 2I) = [up | gate] pre-activation, d_act (L, I) gradient of up * silu(gate)
- * (activations/glu.py:42-43), row_scale (L,) or NULL (a factor on d_act per row: the gate weight of the
- * row's slot), d_h (L, 2I) out = [d_act * silu(gate) | d_act * up * silu'(gate)].  I % 8 == 0.
+ * mi_moe_swiglu_backward, one pass over the sorted rows i = 0..L-1:
+ *   h (L, 2I) = [up | gate] pre-activation, d_act (L, I) = gradient w.r.t. a = up * silu(gate)
+ *   (activations/glu.py:42-43) BEFORE the router weight is applied, i.e. dy[token(i)] @ w_proj[expert(i)];
+ *   g_i = gates[slot(i)] with slot(i) = sorted_scattered[i] (gates NULL: 1; sorted_scattered NULL: slot = i).
+ *   d_h (L, 2I) out = [g d_act * silu(gate) | g d_act * up * silu'(gate)]
+ *   act_g (L, I) out or NULL = g * a               (operand of the down-projection's weight gradient)
+ *   d_gates (T*k) out or NULL: d_gates[slot(i)] = <d_act[i], a[i]>   (= <dy[t], w_proj[e] a>, gradient of the
+ *   router weight; every slot is written exactly once).  I % 8 == 0.
  */
-int mi_moe_swiglu_backward(const void* h, const void* d_act, const void* row_scale, void* d_h, int L, int I,
-                           int dtype, mi_moe_stream_t stream);
+int mi_moe_swiglu_backward(const void* h, const void* d_act, const void* gates, const int32_t* sorted_scattered,
+                           void* d_h, void* act_g, void* d_gates, int L, int I, int dtype, mi_moe_stream_t stream);
 /* d_gates[t, j] = <dy[t, :], o[t*k + j, :]>: the gradient of mi_moe_combine w.r.t. the gates.  H % 8 == 0. */
 int mi_moe_combine_grad_gates(const void* o, const void* dy, void* d_gates, int T, int k, int H, int dtype,
                               mi_moe_stream_t stream);

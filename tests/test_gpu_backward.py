@@ -19,33 +19,51 @@ def _ops():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("L,I", [(1, 8), (37, 64), (513, 512), (4099, 1408)])
-@pytest.mark.parametrize("scaled", [False, True])
-def test_swiglu_backward(device, dtype, L, I, scaled):
+@pytest.mark.parametrize("L,I,k", [(1, 8, 1), (36, 64, 2), (512, 512, 8), (4098, 1408, 6)])
+@pytest.mark.parametrize("routed", [False, True])
+def test_swiglu_backward(device, dtype, L, I, k, routed):
+    """d_h, g * a and the router-weight gradient against autograd through z = sum_i g_i <c_i, up_i * silu(gate_i)>
+    (c = d_act plays the role of the upstream gradient w_proj^T dy)."""
     g = torch.Generator().manual_seed(L * 31 + I)
     h = (torch.randn(L, 2 * I, generator=g) * 2).to(dtype)
     d_act = torch.randn(L, I, generator=g).to(dtype)
-    s = torch.rand(L, generator=g).to(dtype) if scaled else None
+    gates = torch.rand(L // k, k, generator=g).to(dtype) if routed else None
+    ss = torch.randperm(L, generator=g).to(torch.int32) if routed else None
 
     hf = h.float().requires_grad_(True)
     a = hf[:, :I] * F.silu(hf[:, I:])
-    upstream = d_act.float() * (s.float().unsqueeze(-1) if scaled else 1.0)
-    a.backward(upstream)
+    if routed:
+        gf = gates.float().requires_grad_(True)
+        g_rows = gf.reshape(-1)[ss.long()].unsqueeze(-1)
+    else:
+        g_rows = 1.0
+    (g_rows * d_act.float() * a).sum().backward()
 
-    got = _ops().swiglu_backward(h.to(device), d_act.to(device), None if s is None else s.to(device))
-    assert got.dtype == dtype and tuple(got.shape) == (L, 2 * I)
+    d_h, act_g, d_gates = _ops().swiglu_backward(
+        h.to(device), d_act.to(device), None if gates is None else gates.to(device),
+        None if ss is None else ss.to(device), want_act=True, want_gate_grad=routed)
+    assert d_h.dtype == dtype and tuple(d_h.shape) == (L, 2 * I)
     eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
-    torch.testing.assert_close(got.cpu().float(), hf.grad, rtol=2 * eps, atol=1e-6)
+    torch.testing.assert_close(d_h.cpu().float(), hf.grad, rtol=2 * eps, atol=1e-6)
+    torch.testing.assert_close(act_g.cpu().float(), (g_rows * a).detach(), rtol=2 * eps, atol=1e-6)
+    if routed:
+        assert tuple(d_gates.shape) == tuple(gates.shape)
+        torch.testing.assert_close(d_gates.cpu().float(), gf.grad, rtol=2 * eps, atol=2e-4 * I ** 0.5)
+    else:
+        assert d_gates is None
 
 
 def test_swiglu_backward_empty_and_errors(device):
     ops = _ops()
-    out = ops.swiglu_backward(torch.empty(0, 32, device=device, dtype=torch.bfloat16),
-                              torch.empty(0, 16, device=device, dtype=torch.bfloat16))
-    assert tuple(out.shape) == (0, 32)
+    out, act_g, d_gates = ops.swiglu_backward(torch.empty(0, 32, device=device, dtype=torch.bfloat16),
+                                              torch.empty(0, 16, device=device, dtype=torch.bfloat16))
+    assert tuple(out.shape) == (0, 32) and act_g is None and d_gates is None
     with pytest.raises(ValueError):
         ops.swiglu_backward(torch.zeros(4, 30, device=device, dtype=torch.bfloat16),
                             torch.zeros(4, 16, device=device, dtype=torch.bfloat16))
+    with pytest.raises(ValueError):  # the router-weight gradient needs the router weights
+        ops.swiglu_backward(torch.zeros(4, 32, device=device, dtype=torch.bfloat16),
+                            torch.zeros(4, 16, device=device, dtype=torch.bfloat16), want_gate_grad=True)
     from dolomite_engine_amd._lib import MiMoeError
 
     with pytest.raises(MiMoeError):  # fp32 is not a dtype of this kernel
