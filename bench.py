@@ -64,6 +64,11 @@ class StageTimer:
         self.torch.cuda.synchronize()
         return {n: sum(a.elapsed_time(b) for a, b in evs) / len(evs) for n, evs in self.events.items()}
 
+    def per_step(self, steps):
+        """Total time of every stage per step (a stage may run several times in one step)."""
+        self.torch.cuda.synchronize()
+        return {n: sum(a.elapsed_time(b) for a, b in evs) / steps for n, evs in self.events.items()}
+
 
 def build_module(w, inputs, device, fp8_tiled=True):
     import torch
@@ -152,6 +157,10 @@ def main():
                          "(ms_per_step_graph_replay); value / ms_per_step stay the eager module call")
     ap.add_argument("--fp8-row-major", action="store_true",
                     help="decode workload: keep the fp8 expert weights row-major instead of in the streamed-tile layout")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time a training step of the layer (forward + backward for the input and every "
+                         "parameter, synthetic upstream gradient) through the kernel branch and through the eager "
+                         "branch; reported as extra fields, value / ms_per_step stay the forward")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy so that a rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE run of this command contains a kernel of known traffic to scale by")
@@ -231,6 +240,49 @@ def main():
         idx = ops.router_fused(x, m.gate.weight, k, bias=m.router_logit_bias)[2]
         counts = torch.bincount(idx.flatten().long(), minlength=E).cpu()
 
+    train = None
+    if args.backward:
+        if w.fp8:
+            print("bench.py: --backward needs a 16-bit workload", file=sys.stderr)
+            sys.exit(2)
+        from dolomite_engine_amd.loss import clear_aux_loss, get_aux_loss
+
+        m.train()
+        xg = x.clone().requires_grad_(True)
+        dy = torch.randn_like(x)
+
+        def train_step(kernels: bool):
+            m.zero_grad(set_to_none=True)
+            xg.grad = None
+            clear_aux_loss()
+            if kernels:
+                with enable_kernels([Kernel.scattermoe]):
+                    out_ = m(xg)
+            else:
+                out_ = m(xg)
+            ((out_ * dy).sum() + 0.01 * get_aux_loss()).backward()
+
+        train = {}
+        for name, kernels in (("kernels", True), ("eager", False)):
+            torch.cuda.reset_peak_memory_stats()
+            for _ in range(3):
+                train_step(kernels)
+            torch.cuda.synchronize()
+            train["peak_mem_gib_" + name] = torch.cuda.max_memory_allocated() / 2 ** 30
+            n = max(3, args.steps // 5)
+            t0 = time.perf_counter()
+            for _ in range(n):
+                train_step(kernels)
+            torch.cuda.synchronize()
+            train["ms_per_step_fwd_bwd_" + name] = (time.perf_counter() - t0) / n * 1e3
+        timer = StageTimer()
+        ops.set_stage_timer(timer)
+        for _ in range(5):
+            train_step(True)
+        train["stages_ms_fwd_bwd"] = timer.per_step(5)
+        ops.set_stage_timer(None)
+        m.eval()
+
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = T / (elapsed / args.steps)
     flops = 6.0 * L * H * I
@@ -271,6 +323,8 @@ def main():
     }
     if graph_ms is not None:
         out["ms_per_step_graph_replay"] = graph_ms
+    if train is not None:
+        out["training"] = train
     if not args.no_cpu_baseline:
         sample = args.cpu_sample_tokens or min(T, 8192)
         out["cpu_baseline"] = cpu_baseline(w, inputs, sample)
