@@ -43,7 +43,7 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
         half = x.dtype in (torch.float16, torch.bfloat16) and I % 8 == 0
 
         # gradient w.r.t. the SwiGLU output a, in sorted order and before the router weight: dy[t_i] @ w_proj[e_i]
-        d_act = ops.scattered_gemm(dy, w_proj.transpose(1, 2).contiguous(), k, ss, off, False, True)
+        d_act = ops.scattered_gemm(dy, w_proj, k, ss, off, False, True, weight_kn=True)
         # pre-activation recomputed; one pass then gives d_h (with the router weight g_i of the row applied),
         # g_i * a_i for the down-projection's weight gradient, and the gradient of the router weights,
         # <dy[t], w_proj[e] a_i> = <d_act_i, a_i>
@@ -66,7 +66,7 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
         del h, d_act
 
         # gradient w.r.t. x: every slot's contribution in flat-slot order, then the k slots of a token summed
-        dx_slots = ops.scattered_gemm(d_h, w_fc.transpose(1, 2).contiguous(), 1, ss, off, True, False)
+        dx_slots = ops.scattered_gemm(d_h, w_fc, 1, ss, off, True, False, weight_kn=True)
         dx = ops.combine(dx_slots, torch.ones_like(gates))
         del dx_slots
 

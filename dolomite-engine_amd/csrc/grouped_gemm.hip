@@ -666,9 +666,13 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GemmArgs 
 
 #define PERSIST_MAX_E 256
 
-template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool PP>
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool PP, bool WT = false>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(GemmArgs a) {
   static_assert(BK == 32 || BK == 64, "BK");
+  // WT: the expert weights are (K, N) row-major ("x @ W" with W as stored, the form both data gradients of the
+  // backward take).  A K slice of them is 32 rows of 512 bytes; it is staged as it lies in HBM and the fragments
+  // are read with the transposing LDS read (see read_frags).
+  static_assert(!WT || (PP && !GLU && BK == 32 && BNW == 256), "transposed-weight form");
   constexpr int NSTAGE = BK == 32 ? 4 : 2;   // ring of 128 KiB either way
   constexpr int STEPS = BK / 16;             // MFMA k-steps per ring stage
   constexpr int RPI = BK == 32 ? 16 : 8;     // stage rows filled by one DMA instruction (1 KiB)
@@ -813,6 +817,15 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
       if (j < NXLD) {
         const int s = a.gather ? raw[j] / a.kdiv : raw[j];
         ts.off[j] = ((uint32_t)s * (uint32_t)a.K + lchunk * 8) * (uint32_t)sizeof(T);
+      } else if constexpr (WT) {
+        // DMA instruction = two K rows of the slice; LDS piece lane % 32 of row krow holds the logical 16-byte
+        // piece whose 32-byte group is (piece / 2) ^ f(krow): the swizzle the transposing reads expect
+        const int krow = 2 * ((j - NXLD) * NW + wave) + (lane >> 5);
+        const int f = (krow & 3) | (((krow >> 3) & 3) << 2);
+        const int piece = lane & 31;
+        int col = tc.nt * BN + ((((piece >> 1) ^ f) & 15) << 4) + (piece & 1) * 8;
+        if (col > a.N - 8) col = a.N - 8;  // column tail re-reads the last piece of the row; never stored
+        ts.off[j] = ((uint32_t)krow * (uint32_t)a.N + col) * (uint32_t)sizeof(T);
       } else {
         const int wr = ((j - NXLD) * NW + wave) * RPI + (lane >> LROW_SHIFT);
         int col, half = 0;
@@ -831,7 +844,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   auto dma_slice = [&](const TileSrc& cur, const TileSrc& next, bool from_next, int kt, int stage) {
     const size_t kbytes = (size_t)kt * BK * sizeof(T);
     const unsigned char* xs = xbase + kbytes;
-    const unsigned char* ws = (from_next ? next.wbase : cur.wbase) + kbytes;
+    const unsigned char* ws = (from_next ? next.wbase : cur.wbase) + (WT ? kbytes * a.N : kbytes);
     const uint32_t stage_lds = (uint32_t)(size_t)(lds_ptr_t)smem_raw + stage * STAGE_BYTES;
     // activation rows fill stage rows [0, BM), weight rows [BM, BM + BNW)
     auto grp = [&](int j) { return j < NXLD ? (j * NW + wave) : (BM / RPI + (j - NXLD) * NW + wave); };
@@ -870,11 +883,28 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
 
   constexpr int NBUF = PP ? 1 : 2;
   frag_t xf[NBUF][MB], wf[NBUF][NB];
+  // WT: ds_read_b64_tr_b16 transposes 4 rows x 16 columns across 16 lanes: lane i of the group supplies the
+  // address of (row i / 4, columns 4 (i % 4) ..) and receives column i of the four rows.  Lane group q reads rows
+  // 8q .. 8q + 3 and, 2 KiB further, 8q + 4 .. 8q + 7: together the 8 contraction values the matrix instruction
+  // wants from lane (column, q).
+  typedef short tr_s16x4 __attribute__((ext_vector_type(4)));
+  const int tr_i = lane & 15, tr_q = lane >> 4;
+  const uint32_t tr_base = (8 * tr_q + (tr_i >> 2)) * (BNW * 2) + ((((tr_i >> 2) | (tr_q << 2))) << 5) + (tr_i & 3) * 8;
+  const uint32_t lds_base = (uint32_t)(size_t)(lds_ptr_t)smem_raw;
   auto read_frags = [&](int stage, int kk, int buf) {
     const unsigned char* s = smem_raw + stage * STAGE_BYTES + chunk_byte[kk];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-      wf[buf][nb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_w_off[nb]));
+    for (int nb = 0; nb < NB; ++nb) {
+      if constexpr (WT) {
+        typedef __attribute__((address_space(3))) tr_s16x4* tr_ptr_t;
+        const uint32_t addr = lds_base + stage * STAGE_BYTES + BM * BK * 2 + (tr_base ^ ((uint32_t)(wn * NB + nb) << 5));
+        const tr_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(size_t)addr);
+        const tr_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(size_t)(addr + 4 * BNW * 2));
+        wf[buf][nb] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      } else {
+        wf[buf][nb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_w_off[nb]));
+      }
+    }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
       xf[buf][mb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_x_off[mb]));
@@ -1167,12 +1197,12 @@ static int launch_dma(GemmArgs a, hipStream_t s) {
   return mi_launch_status();
 }
 
-template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool PP>
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool PP, bool WT = false>
 static int launch_persistent(GemmArgs a, hipStream_t s) {
   constexpr int BN = GLU ? BNW / 2 : BNW;
   constexpr int NW = WM * WN;
   const size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T) + (PP ? 0 : (size_t)NW * (NW > 4 ? 2048 : 4096)) + (size_t)a.E * 8;
-  auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, BK, PP>;
+  auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, BK, PP, WT>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;
@@ -1278,6 +1308,25 @@ extern "C" int mi_moe_scattered_gemm_cfg(const void* in, const void* w, void* ou
   a.L = L; a.K = K; a.N = N; a.E = E; a.kdiv = k; a.n_tiles = 0;
   a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1;
   return run_gemm(a, dtype, false, cfg, L, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mi_moe_scattered_gemm_wt(const void* in, const void* w_kn, void* out, const int32_t* sorted_scattered,
+                                        const int32_t* expert_offsets, int L, int K, int N, int E, int k,
+                                        int grouped_in, int grouped_out, int dtype, mi_moe_stream_t stream) {
+  int rc = check_common(in, w_kn, out, sorted_scattered, expert_offsets, L, K, N, E, k, dtype,
+                        !grouped_in || !grouped_out);
+  if (rc != MI_MOE_OK) return rc;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (L == 0) return MI_MOE_OK;
+  GemmArgs a;
+  a.in = in; a.w = w_kn; a.out = out;
+  a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
+  a.L = L; a.K = K; a.N = N; a.E = E; a.kdiv = k; a.n_tiles = 0;
+  a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1;
+  if (!tiled_ok(a, L, false) || !persistent_ok(a)) return MI_MOE_EUNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MI_MOE_BF16) return launch_persistent<bf16_t, 256, 256, 4, 2, false, 32, true, true>(a, s);
+  return launch_persistent<f16_t, 256, 256, 4, 2, false, 32, true, true>(a, s);
 }
 
 extern "C" int mi_moe_scattered_gemm(const void* in, const void* w, void* out, const int32_t* sorted_scattered,

@@ -225,15 +225,22 @@ def sort_bin(selected_experts: torch.Tensor, num_experts: int):
 
 
 def scattered_gemm(inputs: torch.Tensor, weight: torch.Tensor, k: int, sorted_scattered_idxs: torch.Tensor,
-                   expert_offsets: torch.Tensor, grouped_in: bool, grouped_out: bool, cfg: int = -1) -> torch.Tensor:
-    """Grouped GEMM with the weight in native (E, out, in) layout; returns (L, out)."""
+                   expert_offsets: torch.Tensor, grouped_in: bool, grouped_out: bool, cfg: int = -1,
+                   weight_kn: bool = False) -> torch.Tensor:
+    """Grouped GEMM with the weight in native (E, out, in) layout; returns (L, out).
+
+    ``weight_kn``: the weight is (E, in, out) instead (``inputs @ weight[e]``, the form of the backward's data
+    gradients).  Shapes the transposed-weight kernel does not take are transposed once and run the normal way."""
     _dev(inputs, weight, sorted_scattered_idxs, expert_offsets)
     _no_grad(inputs, weight)
     inputs = inputs.contiguous()
     weight = weight.contiguous()
     ss = _i32(sorted_scattered_idxs).contiguous()
     off = _i32(expert_offsets).contiguous()
-    E, N, K = weight.shape
+    if weight_kn:
+        E, K, N = weight.shape
+    else:
+        E, N, K = weight.shape
     if inputs.shape[1] != K or weight.dtype != inputs.dtype:
         raise ValueError("inputs must be (rows, in_features) in the dtype of the weights")
     L = ss.numel()
@@ -242,10 +249,20 @@ def scattered_gemm(inputs: torch.Tensor, weight: torch.Tensor, k: int, sorted_sc
     if not grouped_in and inputs.shape[0] * k != L:
         raise ValueError("scattered inputs must have L / k rows")
     out = torch.empty((L, N), dtype=inputs.dtype, device=inputs.device)
+    lib = _lib.load()
+    if weight_kn:
+        with _stage("scattered_gemm"):
+            rc = lib.mi_moe_scattered_gemm_wt(_ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N, E, k,
+                                              int(grouped_in), int(grouped_out), _code(inputs.dtype), _stream())
+        if rc == 0:
+            return out
+        if rc not in (_lib.MI_MOE_EUNSUPPORTED, _lib.MI_MOE_EDTYPE):
+            check(rc)
+        weight = weight.transpose(1, 2).contiguous()
     with _stage("scattered_gemm"):
-        check(_lib.load().mi_moe_scattered_gemm_cfg(_ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N,
-                                                   E, k, int(grouped_in), int(grouped_out), _code(inputs.dtype), cfg,
-                                                   _stream()))
+        check(lib.mi_moe_scattered_gemm_cfg(_ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N,
+                                            E, k, int(grouped_in), int(grouped_out), _code(inputs.dtype), cfg,
+                                            _stream()))
     return out
 
 

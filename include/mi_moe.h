@@ -130,6 +130,17 @@ int mi_moe_scattered_gemm(const void* in, const void* w, void* out, const int32_
                           const int32_t* expert_offsets, int L, int K, int N, int E, int k,
                           int grouped_in, int grouped_out, int dtype, mi_moe_stream_t stream);
 
+/*
+ * The same product with the expert weights stored (E, K, N), i.e. out[orow(i), :] = in[irow(i), :] @ w_kn[e_i]:
+ * the form of both data gradients of the backward of scattered_experts (moe.py:91-101), d_act = dy @ w_proj[e] and
+ * dx = d_h @ w_fc[e], with the weights as the module keeps them (no transposed copy).  F16 / BF16, and only the
+ * shapes the persistent tile kernel takes (K % 32 == 0, K >= 128, N % 8 == 0, E <= 256, 16-byte aligned
+ * pointers); MI_MOE_EUNSUPPORTED otherwise (the caller can transpose and use mi_moe_scattered_gemm).
+ */
+int mi_moe_scattered_gemm_wt(const void* in, const void* w_kn, void* out, const int32_t* sorted_scattered,
+                             const int32_t* expert_offsets, int L, int K, int N, int E, int k, int grouped_in,
+                             int grouped_out, int dtype, mi_moe_stream_t stream);
+
 /* Same call with an explicit kernel configuration (tuning / benchmarking / tests): cfg = -1 picks one
  * from the shape; 0 / 1 / 2 = register-staged 256x256 / 128x128 / 32x256 tiles; 3 = one thread per
  * output element (any shape, the only fp32 path); 4 = DMA-staged 128x128 (K % 32 == 0); 5 / 6 =

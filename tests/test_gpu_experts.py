@@ -76,6 +76,32 @@ def test_scattered_gemm(device, dtype, T, E, k, K, N, mode, cfg):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,E,k,K,N", CASES + [(900, 4, 2, 1024, 1536), (2048, 8, 2, 512, 72)])
+@pytest.mark.parametrize("mode", ["scatter2group", "group2scatter"])
+def test_scattered_gemm_weight_kn(device, dtype, T, E, k, K, N, mode):
+    """Weights stored (E, K, N), as both data gradients of the backward use them: against the oracle, and bit for
+    bit against the native-layout kernel on a transposed copy where the transposed-weight kernel runs (same tile
+    shape, same order of the contraction)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(T * 5 + E + K + N)
+    se, ss, off = _routing(T, E, k, seed=T + E + 1, skew=(T % 2 == 0))
+    L = T * k
+    grouped_in = mode.startswith("group")
+    grouped_out = mode.endswith("group")
+    x = _rand((L if grouped_in else T, K), 1.0, dtype, g)
+    w_kn = _rand((E, K, N), 0.05, dtype, g)
+    print(f"gemm weight_kn {mode} T={T} E={E} k={k} K={K} N={N} {dtype}", flush=True)
+    xd, wd, ssd, offd = x.to(device), w_kn.to(device), ss.to(device), off.to(device)
+    out = ops.scattered_gemm(xd, wd, k, ssd, offd, grouped_in, grouped_out, weight_kn=True)
+    ref = oracle.scattered_experts_oracle(x, w_kn.transpose(1, 2).contiguous(), k, se, ss, off, grouped_in=grouped_in,
+                                          grouped_out=grouped_out)
+    torch.testing.assert_close(out.cpu().float(), ref, **TOL[dtype])
+    if dtype != torch.float32 and K % 32 == 0 and K >= 128 and N % 8 == 0:
+        same = ops.scattered_gemm(xd, wd.transpose(1, 2).contiguous(), k, ssd, offd, grouped_in, grouped_out, cfg=7)
+        assert torch.equal(out, same)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,E,k,H,I", [(15, 8, 8, 32, 128), (512, 8, 2, 256, 512), (333, 5, 2, 136, 100),
                                        (2048, 4, 2, 512, 256), (64, 64, 6, 256, 128)])
 @pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4, 5, 6, 7])
