@@ -51,6 +51,7 @@ struct WgradArgs {
   const int32_t* b_idx;           // same for `b`
   const int32_t* expert_offsets;  // (E,) inclusive ends of the experts' row ranges
   float* partial;                 // [group][M][N]
+  int* next_item;                 // [8] per-XCD work counters, zero on entry
   int L, M, N, E, chunk, m_tiles, n_tiles;
 };
 
@@ -118,6 +119,7 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
   typedef const __attribute__((address_space(4))) int32_t* const_idx_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   int* etab = reinterpret_cast<int*>(smem_raw + NSTAGE * STAGE_BYTES);
+  int* item_slot = etab + 2 * a.E;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
   wgrad_build_table(a.expert_offsets, a.E, a.chunk, etab, lane, wave);
   const int total_groups = etab[2 * (a.E - 1)];
   const int tiles = a.m_tiles * a.n_tiles;
-  const int xcd = blockIdx.x & 7, slot0 = blockIdx.x >> 3, nslot = gridDim.x >> 3;
+  const int xcd = blockIdx.x & 7;
 
   // An expert with n rows has ceil(n / chunk) groups of equal size (a multiple of 32 rows, the last one shorter).
   auto group_rows = [&](int n, int groups) { return ((n + groups - 1) / groups + 31) & ~31; };
@@ -182,7 +184,14 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
   const int fl = (fi >> 2) | (fq << 2);
   const uint32_t frag_base = (8 * fq + (fi >> 2)) * (TILE * 2) + (fl << 5) + (fi & 3) * 8;
 
-  for (int item = slot0; item < items_x; item += nslot) {
+  // Items of an XCD are handed out in order through a counter: the workgroups of the XCD stay on neighbouring
+  // items (same group of rows, shared through the L2) and none of them idles while another still has a queue.
+  for (;;) {
+    if (tid == 0) *item_slot = atomicAdd(a.next_item + xcd, 1);
+    __syncthreads();
+    const int item = __builtin_amdgcn_readfirstlane(*item_slot);
+    __syncthreads();
+    if (item >= items_x) break;
     const int grp = gbeg + item / tiles;
     const int tile = item % tiles;
     const int mt = tile % a.m_tiles, nt = tile / a.m_tiles;
@@ -338,6 +347,10 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
   }
 }
 
+__global__ void wgrad_zero_counters_kernel(int* counters) {
+  if (threadIdx.x < 8) counters[threadIdx.x] = 0;
+}
+
 // dW[e] = sum of expert e's partial slabs in group order, rounded once; zeros for an expert without rows
 template <typename T>
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ partial,
@@ -384,7 +397,8 @@ static long wgrad_max_groups(int L, int E, int chunk) { return (long)L / chunk +
 
 extern "C" size_t mi_moe_grouped_wgrad_workspace_bytes(int L, int E, int M, int N) {
   if (L < 1 || E < 1 || M < 1 || N < 1) return 0;
-  return (size_t)wgrad_max_groups(L, E, wgrad_chunk(L, M, N)) * (size_t)M * (size_t)N * sizeof(float);
+  // [partial slabs][8 work counters, padded to 256 bytes]
+  return (size_t)wgrad_max_groups(L, E, wgrad_chunk(L, M, N)) * (size_t)M * (size_t)N * sizeof(float) + 256;
 }
 
 extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const void* b, const int32_t* b_idx,
@@ -406,11 +420,17 @@ extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const v
   WgradArgs g;
   g.a = a; g.b = b; g.a_idx = a_idx; g.b_idx = b_idx; g.expert_offsets = expert_offsets;
   g.partial = static_cast<float*>(workspace);
+  g.next_item = nullptr;
   g.L = L; g.M = M; g.N = N; g.E = E;
   g.chunk = wgrad_chunk(L, M, N);
+  if (L > 0) {
+    g.next_item = reinterpret_cast<int*>(static_cast<unsigned char*>(workspace) +
+                                         (size_t)wgrad_max_groups(L, E, g.chunk) * (size_t)M * (size_t)N * sizeof(float));
+    hipLaunchKernelGGL(wgrad_zero_counters_kernel, dim3(1), dim3(64), 0, s, g.next_item);
+  }
   g.m_tiles = mi_ceil_div(M, 256);
   g.n_tiles = mi_ceil_div(N, 256);
-  const size_t lds = 4 * 2 * 32 * 256 * 2 + (size_t)E * 8;
+  const size_t lds = 4 * 2 * 32 * 256 * 2 + (size_t)E * 8 + 16;
   int dev = 0, cus = 0;
   hipError_t e;
   if ((e = hipGetDevice(&dev)) != hipSuccess) return (int)e;
