@@ -46,6 +46,9 @@ SIGNATURES: dict[str, tuple] = {
     "mi_moe_combine_grad_gates": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mi_moe_grouped_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mi_moe_grouped_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "mi_moe_aux_loss_workspace_bytes": (_sz, [_i, _i]),
+    "mi_moe_aux_loss": (_i, [_vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
+    "mi_moe_aux_loss_backward": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "mi_moe_fp8_tiled_bytes": (_sz, [_i, _i, _i, _i]),
     "mi_moe_up_swiglu_fp8": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mi_moe_down_fp8": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),

@@ -88,3 +88,19 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
                     d_w_proj[e] = dy[t_e].t() @ act_g[rows]
                 start = end
         return dx, d_w_fc, d_w_proj, d_gates, None, None, None
+
+
+class SwitchAuxLoss(torch.autograd.Function):
+    """The router's auxiliary loss (moe.py:346-369, one data-parallel rank) as two fused passes over the logits:
+    value in the forward, gradient w.r.t. the logits in the backward.  Returns a 0-d tensor in the logits' dtype."""
+
+    @staticmethod
+    def forward(ctx, logits, topk_idxs):
+        loss_w = ops.aux_loss(logits.detach(), topk_idxs)
+        ctx.save_for_backward(logits, loss_w)
+        return loss_w[0].to(logits.dtype)
+
+    @staticmethod
+    def backward(ctx, grad):
+        logits, loss_w = ctx.saved_tensors
+        return ops.aux_loss_backward(logits.detach(), loss_w, grad), None

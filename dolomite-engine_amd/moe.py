@@ -13,8 +13,10 @@ this package (router -> sort/bin -> grouped up-projection with fused SwiGLU -> g
 down-projection -> gate-weighted combine).  Without it the eager torch branch runs, which is the
 reference's own eager branch (moe.py:292-307) and works on any device.
 
-The kernel branch is forward-only (inference): it refuses tensors that require grad while grad
-mode is on, and it raises if the kernel library is missing -- it never falls back silently.
+With the SwiGLU activation the kernel branch also trains: when a gradient is needed the experts run through
+``autograd.ScatteredSwiGLUExperts`` and the auxiliary loss through ``autograd.SwitchAuxLoss``.  With any other
+activation it is forward-only and refuses tensors that require grad while grad mode is on.  It raises if the kernel
+library is missing -- it never falls back silently.
 """
 
 from __future__ import annotations
@@ -27,7 +29,7 @@ import torch.nn.functional as F
 
 from . import ops
 from .activations import GLUActivation, get_activation_function, is_glu
-from .autograd import ScatteredSwiGLUExperts
+from .autograd import ScatteredSwiGLUExperts, SwitchAuxLoss
 from .enums import Kernel
 from .kernels import is_kernel_allowed
 from .linear import ParameterizedLinear
@@ -280,13 +282,16 @@ class MoE(nn.Module):
             if residual is not None:
                 hidden_states = hidden_states + residual.reshape(hidden_states.shape)
 
-        aux_loss = (
-            self._compute_switch_loss(
+        if not self.training:
+            aux_loss = 0
+        elif is_kernel_allowed(Kernel.scattermoe) and ops.aux_loss_supported(router_logits.view(-1, self.num_experts)):
+            # both passes over the (T, E) logits fused (fp32 arithmetic; the eager line below rounds its
+            # intermediates to the model dtype)
+            aux_loss = SwitchAuxLoss.apply(router_logits.view(-1, self.num_experts), selected_experts)
+        else:
+            aux_loss = self._compute_switch_loss(
                 logits=router_logits, probs=torch.softmax(router_logits, dim=-1), topk_idxs=selected_experts
             )
-            if self.training
-            else 0
-        )
         add_aux_loss(aux_loss)
 
         return hidden_states

@@ -6,8 +6,9 @@ moe.py:40 and moe.py:91-101), so either can be bound in their place.  The remain
 the fused stages the MoE module of this package calls.
 
 PyTorch is used for device memory and the current stream only; every function enqueues HIP
-kernels on ``torch.cuda.current_stream()`` and returns without synchronising.  All of this is
-forward-only: tensors that require grad are refused while grad mode is on.
+kernels on ``torch.cuda.current_stream()`` and returns without synchronising.  None of these functions
+records a gradient: tensors that require grad are refused while grad mode is on (the differentiable
+compositions are in ``autograd.py``).
 """
 
 from __future__ import annotations
@@ -78,7 +79,8 @@ def _dev(*tensors: torch.Tensor | None) -> None:
 def _no_grad(*tensors: torch.Tensor | None) -> None:
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
         raise RuntimeError(
-            "the MI355X scattermoe kernels are forward-only: run under torch.no_grad() / inference_mode()"
+            "the MI355X scattermoe kernels are forward-only (they record no gradient): run under torch.no_grad() / "
+            "inference_mode(), or go through the module / autograd.py"
         )
 
 
@@ -390,6 +392,48 @@ def grouped_wgrad(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor
                                        _ptr(ws), ws_bytes, L, a.shape[0], b.shape[0], M, N, E, _code(a.dtype),
                                        _stream()))
     return dw
+
+
+def aux_loss_supported(logits: torch.Tensor) -> bool:
+    return logits.is_cuda and logits.dim() == 2 and logits.shape[0] >= 1 and 1 <= logits.shape[1] <= 256 and \
+        logits.dtype in (torch.float32, torch.float16, torch.bfloat16)
+
+
+def aux_loss(logits: torch.Tensor, topk_idxs: torch.Tensor) -> torch.Tensor:
+    """Switch + z auxiliary loss of moe.py:346-369 (single data-parallel rank) from the (T, E) logits and the
+    (T, k) selected experts.  Returns 1 + E floats: [0] the loss, [1:] d loss / d (summed probabilities), which
+    :func:`aux_loss_backward` takes."""
+    _dev(logits, topk_idxs)
+    _no_grad(logits)
+    logits = logits.contiguous()
+    idx = _i32(topk_idxs).contiguous()
+    T, E = logits.shape
+    if idx.dim() != 2 or idx.shape[0] != T:
+        raise ValueError("topk_idxs must be (T, k)")
+    lib = _lib.load()
+    ws_bytes = int(lib.mi_moe_aux_loss_workspace_bytes(T, E))
+    ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=logits.device)
+    loss_w = torch.empty(1 + E, dtype=torch.float32, device=logits.device)
+    with _stage("aux_loss"):
+        check(lib.mi_moe_aux_loss(_ptr(logits), _ptr(idx), _ptr(loss_w), _ptr(ws), ws_bytes, T, E, idx.shape[1],
+                                  _code(logits.dtype), _stream()))
+    return loss_w
+
+
+def aux_loss_backward(logits: torch.Tensor, loss_w: torch.Tensor, grad: torch.Tensor) -> torch.Tensor:
+    """Gradient of :func:`aux_loss` w.r.t. the logits, scaled by the scalar ``grad``."""
+    _dev(logits, loss_w, grad)
+    _no_grad(logits)
+    logits = logits.contiguous()
+    T, E = logits.shape
+    if loss_w.dtype != torch.float32 or loss_w.numel() != 1 + E:
+        raise ValueError("loss_w must be the 1 + E floats aux_loss returned")
+    grad = grad.detach().to(torch.float32).reshape(1).contiguous()
+    d_logits = torch.empty_like(logits)
+    with _stage("aux_loss_backward"):
+        check(_lib.load().mi_moe_aux_loss_backward(_ptr(logits), _ptr(loss_w.contiguous()), _ptr(grad), _ptr(d_logits),
+                                                   T, E, _code(logits.dtype), _stream()))
+    return d_logits
 
 
 def scattered_experts(inputs: torch.Tensor, expert_weights: torch.Tensor, k: int,

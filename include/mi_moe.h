@@ -226,6 +226,21 @@ int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const void* b, con
                          int L, int a_rows, int b_rows, int M, int N, int E, int dtype, mi_moe_stream_t stream);
 
 /*
+ * Training-mode auxiliary loss of the router, moe.py:346-369 (one data-parallel rank), and its gradient:
+ *   loss = E * sum_e normalize1(A)_e * normalize1(f)_e + 0.1 * mean_t(logsumexp(logits[t, :])^2),
+ *   A_e = sum_t softmax(logits[t, :])_e,  f_e = occurrences of expert e in topk_idx (T, k).
+ * logits (T, E) of `dtype` (F32 / F16 / BF16), fp32 arithmetic, E <= 256.  Deterministic (fixed-order sums).
+ *   loss_w (1 + E floats) out: [0] the loss, [1 + e] d loss / d A_e (what the backward needs).
+ * mi_moe_aux_loss_backward: d_logits (T, E) of `dtype` = grad[0] * d loss / d logits; `grad` is one float in
+ * device memory (the gradient of the scalar loss).
+ */
+size_t mi_moe_aux_loss_workspace_bytes(int T, int E);
+int mi_moe_aux_loss(const void* logits, const int32_t* topk_idx, float* loss_w, void* workspace, size_t workspace_bytes,
+                    int T, int E, int k, int dtype, mi_moe_stream_t stream);
+int mi_moe_aux_loss_backward(const void* logits, const float* loss_w, const float* grad, void* d_logits, int T, int E,
+                             int dtype, mi_moe_stream_t stream);
+
+/*
  * Decode-shape variants with fp8 (OCP e4m3fn) expert weights and one fp32 scale per output channel.
  * No counterpart in the reference (its fp8 support wraps nn.Linear only, lm_engine/fp8.py:63-73);
  * semantics = dequantise (w * scale[:, None]) then the two calls above.

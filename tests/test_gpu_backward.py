@@ -164,3 +164,49 @@ def test_grouped_wgrad_no_rows(device):
     b = torch.empty(0, 8, dtype=torch.bfloat16, device=device)
     out = ops.grouped_wgrad(a, b, torch.zeros(4, dtype=torch.int32, device=device))
     assert tuple(out.shape) == (4, 16, 8) and not out.any()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k", [(1, 4, 1), (15, 8, 8), (300, 40, 8), (1000, 64, 6), (129, 130, 2), (4100, 256, 3)])
+def test_aux_loss_and_gradient(device, dtype, T, E, k):
+    """Value against the oracle's restatement of moe.py:346-369 on the same (rounded) logits, gradient against
+    autograd through that restatement; both in fp32, so only the summation order differs."""
+    from oracle import moe_oracle as oracle
+
+    g = torch.Generator().manual_seed(T + E * 7 + k)
+    logits = (torch.randn(T, E, generator=g) * 1.5).to(dtype)
+    idx = torch.rand(T, E, generator=g).argsort(dim=1)[:, :k].contiguous()
+    ops = _ops()
+
+    lf = logits.float().clone().requires_grad_(True)
+    ref = oracle.switch_aux_loss(lf, idx)
+    upstream = 0.37
+    (ref * upstream).backward()
+
+    loss_w = ops.aux_loss(logits.to(device), idx.to(device))
+    assert loss_w.dtype == torch.float32 and tuple(loss_w.shape) == (1 + E,)
+    torch.testing.assert_close(loss_w[0].cpu(), ref.detach(), rtol=2e-5, atol=1e-6)
+    d = ops.aux_loss_backward(logits.to(device), loss_w, torch.tensor(upstream, device=device))
+    assert d.dtype == dtype and tuple(d.shape) == (T, E)
+    eps = {torch.float32: 2e-5, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+    # entries are O(1 / T); compare relative to the largest one
+    scale = lf.grad.abs().max()
+    torch.testing.assert_close(d.cpu().float() / scale, lf.grad / scale, rtol=2 * eps, atol=2 * eps)
+    # deterministic
+    assert torch.equal(ops.aux_loss(logits.to(device), idx.to(device)), loss_w)
+
+
+def test_aux_loss_autograd_function(device):
+    from dolomite_engine_amd.autograd import SwitchAuxLoss
+    from oracle import moe_oracle as oracle
+
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(200, 16, generator=g)
+    idx = torch.rand(200, 16, generator=g).argsort(dim=1)[:, :4].contiguous()
+    a = logits.clone().to(device).requires_grad_(True)
+    loss = SwitchAuxLoss.apply(a, idx.to(device))
+    assert loss.dim() == 0 and loss.dtype == torch.float32
+    (loss * 2.0).backward()
+    b = logits.clone().requires_grad_(True)
+    (oracle.switch_aux_loss(b, idx) * 2.0).backward()
+    torch.testing.assert_close(a.grad.cpu(), b.grad, rtol=1e-4, atol=1e-8)

@@ -297,7 +297,8 @@ def test_training_gradients_match_eager_branch(device, dtype, tol, shared):
     y_e, aux_e, dx_e, g_e = run(False)
     y_k, aux_k, dx_k, g_k = run(True)
     torch.testing.assert_close(y_k.float(), y_e.float(), **tol)
-    torch.testing.assert_close(aux_k.float(), aux_e.float(), rtol=1e-4, atol=1e-5)
+    # the kernel branch computes the aux loss in fp32, the eager branch in the model dtype
+    torch.testing.assert_close(aux_k.float(), aux_e.float(), rtol=1e-4 if dtype == torch.float32 else 2e-2, atol=1e-5)
     # relative to the largest entry, like the parameter gradients below
     dx_scale = dx_e.float().abs().max().clamp_min(1e-6)
     torch.testing.assert_close(dx_k.float() / dx_scale, dx_e.float() / dx_scale, rtol=tol["rtol"], atol=tol["rtol"] / 4)
