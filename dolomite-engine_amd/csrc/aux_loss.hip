@@ -5,8 +5,9 @@
 //   A_e = sum_t softmax(logits[t])_e,  f_e = number of (token, slot) pairs routed to expert e,  eps = 1e-12
 //
 // Forward: one pass over the (T, E) logits -- a wave per row computes the row's logsumexp and probabilities
-// and keeps per-lane sums; a workgroup writes one partial row [A (E) | f (E) | sum lse^2]; a one-workgroup
-// second kernel adds the partials in index order (deterministic), forms the loss and w_e = d loss / d A_e.
+// and keeps per-lane sums; a workgroup writes one partial per column [A (E) | f (E) | sum lse^2]; a second kernel
+// adds each column's partials in a fixed order (deterministic) and a third, one workgroup, forms the loss and
+// w_e = d loss / d A_e.
 // Backward: d logits[t, j] = g * p_tj * ( w_j - sum_e p_te w_e  +  0.2 / T * lse_t ), one more pass.
 // All arithmetic in fp32 from the logits as stored; the eager module rounds its intermediates to the model
 // dtype instead, so the two agree to that dtype's rounding, not bit for bit.
@@ -72,33 +73,40 @@ __global__ __launch_bounds__(256) void aux_loss_partial_kernel(const T* __restri
     if (lane + 64 * i < E) acc[wave][lane + 64 * i] = a[i];
   if (lane == 0) zsum[wave] = z;
   __syncthreads();
-  float* out = partial + (size_t)blockIdx.x * (2 * E + 1);
+  // partial[column][block], columns = [A (E) | f (E) | sum lse^2]
+  float* out = partial + blockIdx.x;
+  const size_t nb = gridDim.x;
   for (int e = threadIdx.x; e < E; e += 256) {
-    out[e] = ((acc[0][e] + acc[1][e]) + acc[2][e]) + acc[3][e];
-    out[E + e] = (float)cnt[e];
+    out[e * nb] = ((acc[0][e] + acc[1][e]) + acc[2][e]) + acc[3][e];
+    out[(E + e) * nb] = (float)cnt[e];
   }
-  if (threadIdx.x == 0) out[2 * E] = ((zsum[0] + zsum[1]) + zsum[2]) + zsum[3];
+  if (threadIdx.x == 0) out[2 * E * nb] = ((zsum[0] + zsum[1]) + zsum[2]) + zsum[3];
+}
+
+// column sums of the partials: a wave per column, lanes stride over the blocks, then a fixed butterfly -- the same
+// order every run
+__global__ __launch_bounds__(256) void aux_loss_colsum_kernel(const float* __restrict__ partial, float* __restrict__ colsum,
+                                                              int nblocks, int ncols) {
+  const int lane = threadIdx.x & 63;
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (c >= ncols) return;
+  float s = 0.f;
+  for (int b = lane; b < nblocks; b += 64) s += partial[(size_t)c * nblocks + b];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, MI_WAVE);
+  if (lane == 0) colsum[c] = s;
 }
 
 // loss_w[0] = loss, loss_w[1 + e] = d loss / d A_e
-__global__ __launch_bounds__(256) void aux_loss_finish_kernel(const float* __restrict__ partial, float* __restrict__ loss_w,
-                                                              int nblocks, int Trows, int E) {
+__global__ __launch_bounds__(256) void aux_loss_finish_kernel(const float* __restrict__ colsum, float* __restrict__ loss_w,
+                                                              int Trows, int E) {
   __shared__ float A[AUX_MAX_E], F[AUX_MAX_E];
   __shared__ float scal[4];
-  const int stride = 2 * E + 1;
-  // a wave per column: the lanes stride over the partial rows, then a fixed butterfly -- the same order every run
-  const int lane = threadIdx.x & 63;
-  for (int c = threadIdx.x >> 6; c < stride; c += 4) {
-    float s = 0.f;
-    for (int b = lane; b < nblocks; b += 64) s += partial[(size_t)b * stride + c];
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, MI_WAVE);
-    if (lane == 0) {
-      if (c < E) A[c] = s;
-      else if (c < 2 * E) F[c - E] = s;
-      else scal[3] = s;
-    }
+  for (int e = threadIdx.x; e < E; e += 256) {
+    A[e] = colsum[e];
+    F[e] = colsum[E + e];
   }
+  if (threadIdx.x == 0) scal[3] = colsum[2 * E];
   __syncthreads();
   if (threadIdx.x == 0) {
     float sa = 0.f, sf = 0.f, dot = 0.f;
@@ -150,7 +158,8 @@ static int aux_blocks(int T) { return mi_ceil_div(T, AUX_ROWS_PER_BLOCK); }
 
 extern "C" size_t mi_moe_aux_loss_workspace_bytes(int T, int E) {
   if (T < 1 || E < 1) return 0;
-  return (size_t)aux_blocks(T) * (2 * (size_t)E + 1) * sizeof(float);
+  // [partials: (2E + 1) columns x blocks][column sums: 2E + 1]
+  return ((size_t)aux_blocks(T) + 1) * (2 * (size_t)E + 1) * sizeof(float);
 }
 
 template <typename T>
@@ -159,7 +168,10 @@ static void aux_forward_launch(const void* logits, const int32_t* idx, float* ws
   const int nb = aux_blocks(Trows);
   hipLaunchKernelGGL((aux_loss_partial_kernel<T>), dim3(nb), dim3(256), 0, s, static_cast<const T*>(logits), idx, ws,
                      Trows, E, k);
-  hipLaunchKernelGGL(aux_loss_finish_kernel, dim3(1), dim3(256), 0, s, ws, loss_w, nb, Trows, E);
+  const int ncols = 2 * E + 1;
+  float* colsum = ws + (size_t)nb * ncols;
+  hipLaunchKernelGGL(aux_loss_colsum_kernel, dim3(mi_ceil_div(ncols, 4)), dim3(256), 0, s, ws, colsum, nb, ncols);
+  hipLaunchKernelGGL(aux_loss_finish_kernel, dim3(1), dim3(256), 0, s, colsum, loss_w, Trows, E);
 }
 
 extern "C" int mi_moe_aux_loss(const void* logits, const int32_t* topk_idx, float* loss_w, void* workspace,
