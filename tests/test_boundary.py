@@ -169,7 +169,7 @@ def test_eager_branch_equals_oracle_and_handles_3d_input():
 
 
 def test_tiny_config_full_size_eager_equals_oracle():
-    """BASELINE config 1 (512 tokens, hidden 256, 8 experts, top-2, intermediate 512, fp32) on the CPU."""
+    """The CPU-runnable benchmark configuration (512 tokens, hidden 256, 8 experts, top-2, intermediate 512, fp32) on the CPU."""
     w = oracle.WORKLOADS["tiny-fp32"]
     inp = oracle.make_inputs(w)
     m = _moe(hidden_size=w.H, intermediate_size=w.I, num_experts=w.E, num_experts_per_tok=w.k,
