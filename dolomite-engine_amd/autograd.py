@@ -90,6 +90,78 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
         return dx, d_w_fc, d_w_proj, d_gates, None, None, None
 
 
+class ScatteredExperts(torch.autograd.Function):
+    """One grouped GEMM of the layer with a gradient: the differentiable form of ``ops.scattered_experts``
+    (the reference's external op is differentiable too, moe.py:91-101), for expert MLPs whose activation is not the
+    fused SwiGLU.
+
+        out[orow(i)] = x[irow(i)] @ w[e_i]^T           i = sorted row, w (E, N, K)
+        irow(i) = i (grouped_in) or sorted_scattered[i] // k;   orow(i) = i (grouped_out) or sorted_scattered[i]
+        with gates (T, kg):  y[t] = sum_j gates[t, j] * out[t * kg + j]
+
+    Backward: d x from the transposed-weight form of the same kernel, d w from the grouped weight-gradient kernel
+    (16-bit dtypes; otherwise one library GEMM per expert), d gates from the recomputed rows."""
+
+    @staticmethod
+    def forward(ctx, x, w, k, sorted_scattered, expert_offsets, gates, grouped_in, grouped_out):
+        out = ops.scattered_gemm(x, w, k, sorted_scattered, expert_offsets, grouped_in, grouped_out)
+        if gates is not None:
+            out = ops.combine(out, gates.to(out.dtype))
+        ctx.save_for_backward(x, w, sorted_scattered, expert_offsets, gates)
+        ctx.cfg = (k, grouped_in, grouped_out)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        x, w, ss, off, gates = ctx.saved_tensors
+        k, grouped_in, grouped_out = ctx.cfg
+        E, N, K = w.shape
+        L = ss.numel()
+        d_out = d_out.contiguous()
+        half = x.dtype in (torch.float16, torch.bfloat16)
+        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+
+        d_gates = None
+        if gates is not None:
+            T, kg = gates.shape
+            if ctx.needs_input_grad[5]:
+                rows = ops.scattered_gemm(x, w, k, ss, off, grouped_in, False)
+                if half and N % 8 == 0:
+                    d_gates = ops.combine_grad_gates(rows, d_out, kg).to(gates.dtype)
+                else:
+                    d_gates = torch.bmm(rows.view(T, kg, N), d_out.unsqueeze(-1)).squeeze(-1).to(gates.dtype)
+                del rows
+            # gradient of the (L, N) rows in flat-slot order
+            d_out = (gates.to(d_out.dtype).unsqueeze(-1) * d_out.unsqueeze(1)).reshape(L, N)
+
+        dx = None
+        if need_x:
+            # row i: d_out[orow(i)] @ w[e_i], delivered to irow(i) (kept per slot first when a token fans out to k)
+            dx = ops.scattered_gemm(d_out, w, 1, ss, off, grouped_out, grouped_in, weight_kn=True)
+            if not grouped_in and k > 1:
+                dx = ops.combine(dx, torch.ones((L // k, k), dtype=dx.dtype, device=dx.device)) if half \
+                    else dx.view(L // k, k, K).sum(dim=1)
+
+        dw = None
+        if need_w:
+            ssl = ss.long()
+            a_idx = None if grouped_out else ss.to(torch.int32)
+            b_idx = None if grouped_in else torch.div(ss, k, rounding_mode="floor").to(torch.int32)
+            if half and ops.grouped_wgrad_supported(d_out, x, E):
+                dw = ops.grouped_wgrad(d_out, x, off, a_idx, b_idx)
+            else:
+                dw = torch.zeros_like(w)
+                start = 0
+                for e, end in enumerate(off.tolist()):
+                    if end > start:
+                        rows = torch.arange(start, end, device=x.device)
+                        a = d_out[rows if a_idx is None else ssl[rows]]
+                        b = x[rows if b_idx is None else torch.div(ssl[rows], k, rounding_mode="floor")]
+                        dw[e] = a.t() @ b
+                    start = end
+        return dx, dw, None, None, None, d_gates, None, None
+
+
 class SwitchAuxLoss(torch.autograd.Function):
     """The router's auxiliary loss (moe.py:346-369, one data-parallel rank) as two fused passes over the logits:
     value in the forward, gradient w.r.t. the logits in the backward.  Returns a 0-d tensor in the logits' dtype."""

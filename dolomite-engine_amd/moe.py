@@ -13,9 +13,9 @@ this package (router -> sort/bin -> grouped up-projection with fused SwiGLU -> g
 down-projection -> gate-weighted combine).  Without it the eager torch branch runs, which is the
 reference's own eager branch (moe.py:292-307) and works on any device.
 
-With the SwiGLU activation the kernel branch also trains: when a gradient is needed the experts run through
-``autograd.ScatteredSwiGLUExperts`` and the auxiliary loss through ``autograd.SwitchAuxLoss``.  With any other
-activation it is forward-only and refuses tensors that require grad while grad mode is on.  It raises if the kernel
+The kernel branch also trains: when a gradient is needed a SwiGLU layer runs its experts through
+``autograd.ScatteredSwiGLUExperts``, any other activation through the differentiable ``ops.scattered_experts``
+(``autograd.ScatteredExperts``), and the auxiliary loss through ``autograd.SwitchAuxLoss``.  It raises if the kernel
 library is missing -- it never falls back silently.
 """
 

@@ -448,9 +448,17 @@ def scattered_experts(inputs: torch.Tensor, expert_weights: torch.Tensor, k: int
     (T, out); ``combine_tail`` = (shared, residual, residual_scale) is an extension handed on to
     :func:`combine`."""
     del sorted_expert_idxs
-    w = _native_weight(expert_weights)
     if gates is not None and grouped_out:
         raise ValueError("gates need the output in flat-slot order (grouped_out=False)")
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (inputs, expert_weights, gates)):
+        # like the reference's op this one is differentiable; the gradient lives in autograd.py
+        if combine_tail is not None:
+            raise ValueError("combine_tail is an inference-only fusion")
+        from .autograd import ScatteredExperts
+
+        return ScatteredExperts.apply(inputs, expert_weights.permute(0, 2, 1), k, _i32(sorted_scattered_idxs),
+                                      _i32(expert_offsets), gates, grouped_in, grouped_out)
+    w = _native_weight(expert_weights)
     out = scattered_gemm(inputs, w, k, sorted_scattered_idxs, expert_offsets, grouped_in, grouped_out)
     if combine_tail is not None and gates is None:
         raise ValueError("combine_tail needs gates")

@@ -210,3 +210,43 @@ def test_aux_loss_autograd_function(device):
     b = logits.clone().requires_grad_(True)
     (oracle.switch_aux_loss(b, idx) * 2.0).backward()
     torch.testing.assert_close(a.grad.cpu(), b.grad, rtol=1e-4, atol=1e-8)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mode", ["scatter2group", "group2scatter", "scatter2scatter", "group2group"])
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("T,E,k,K,N", [(40, 4, 2, 64, 48), (300, 6, 3, 256, 264)])
+def test_scattered_experts_is_differentiable(device, dtype, mode, gated, T, E, k, K, N):
+    """ops.scattered_experts with tensors that require grad: value and gradients (inputs, expert weights, gates)
+    against autograd through the oracle's fp32 restatement of the call."""
+    from oracle import moe_oracle as oracle
+
+    grouped_in, grouped_out = mode.startswith("group"), mode.endswith("group")
+    if gated and grouped_out:
+        pytest.skip("gates contract the flat-slot order")
+    g = torch.Generator().manual_seed(T + K + N)
+    sel = torch.rand(T, E, generator=g).argsort(dim=1)[:, :k]
+    se, ss, off = oracle.sort_bin(sel, E)
+    L = T * k
+    x0 = torch.randn(L if grouped_in else T, K, generator=g).to(dtype)
+    w0 = (torch.randn(E, N, K, generator=g) * 0.1).to(dtype)        # native (E, out, in)
+    g0 = torch.rand(T, k, generator=g).to(dtype) if gated else None
+    up = torch.randn(T if gated else L, N, generator=g).to(dtype)
+
+    xr, wr = x0.float().clone().requires_grad_(True), w0.float().clone().requires_grad_(True)
+    gr = g0.float().clone().requires_grad_(True) if gated else None
+    ref = oracle.scattered_experts_oracle(xr, wr, k, se, ss, off, gates=gr, grouped_in=grouped_in, grouped_out=grouped_out)
+    (ref * up.float()).sum().backward()
+
+    ops = _ops()
+    xd, wd = x0.to(device).requires_grad_(True), w0.to(device).requires_grad_(True)
+    gd = g0.to(device).requires_grad_(True) if gated else None
+    out = ops.scattered_experts(xd, wd.permute(0, 2, 1), k, se.to(device), ss.to(device), off.to(device), gates=gd,
+                                grouped_in=grouped_in, grouped_out=grouped_out)
+    (out * up.to(device)).sum().backward()
+
+    tol = dict(rtol=2e-3, atol=2e-4) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+    torch.testing.assert_close(out.detach().cpu().float(), ref.detach(), **tol)
+    for name, got, want in (("x", xd.grad, xr.grad), ("w", wd.grad, wr.grad)) + ((("gates", gd.grad, gr.grad),) if gated else ()):
+        scale = want.abs().max().clamp_min(1e-6)
+        torch.testing.assert_close(got.cpu().float() / scale, want / scale, rtol=tol["rtol"], atol=tol["rtol"]), name

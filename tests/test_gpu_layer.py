@@ -249,32 +249,35 @@ def test_layer_under_hip_graph_capture(device, name, T):
             assert torch.equal(static_y, eager), f"replay {i}"
 
 
-def test_kernel_branch_refuses_grad_without_swiglu(device):
-    """Only the SwiGLU path has a backward; other activations on the kernel branch stay forward-only and say so."""
-    from dolomite_engine_amd import Kernel, MoE, enable_kernels
+def test_low_level_ops_record_no_gradient(device):
+    """The tensor-level kernel wrappers are not differentiable and say so (the differentiable compositions are
+    the module and autograd.py)."""
+    from dolomite_engine_amd import ops
 
-    m = MoE(hidden_size=64, intermediate_size=64, shared_intermediate_size=None, num_experts=4,
-            num_experts_per_tok=2, activation_function="gelu_pytorch_tanh", add_bias=False, dropout=0.0,
-            init_method="normal", initializer_range=0.02, m_width=None, num_layers=1,
-            use_padding_free_transformer=True)
-    m = m.to(torch.bfloat16).to(device).eval()
-    x = torch.randn(8, 64, device=device, dtype=torch.bfloat16)
-    with enable_kernels([Kernel.scattermoe]):
-        with pytest.raises(RuntimeError, match="forward-only"):
-            m(x)
+    x = torch.randn(8, 64, device=device, dtype=torch.bfloat16, requires_grad=True)
+    w = torch.randn(4, 32, 64, device=device, dtype=torch.bfloat16)
+    ss = torch.arange(8, device=device, dtype=torch.int32)
+    off = torch.tensor([2, 4, 6, 8], device=device, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="forward-only"):
+        ops.scattered_gemm(x, w, 1, ss, off, False, True)
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, dict(rtol=2e-3, atol=2e-5)), (torch.bfloat16, dict(rtol=5e-2, atol=2e-2))])
 @pytest.mark.parametrize("shared", [None, 64])
-def test_training_gradients_match_eager_branch(device, dtype, tol, shared):
+@pytest.mark.parametrize("activation", ["swiglu", "gelu_pytorch_tanh", "geglu"])
+def test_training_gradients_match_eager_branch(device, dtype, tol, shared, activation):
     """Training through the kernel branch: output, aux loss and every gradient (input, router, both expert
-    weight tensors, shared experts) against torch autograd through the eager branch of the same module."""
+    weight tensors, shared experts) against torch autograd through the eager branch of the same module.
+    swiglu takes the fused expert function, the other activations the differentiable scattered_experts with the
+    activation in torch between the two grouped GEMMs."""
     from dolomite_engine_amd import Kernel, MoE, enable_kernels
     from dolomite_engine_amd.loss import clear_aux_loss, get_aux_loss
 
+    if activation != "swiglu" and shared is not None:
+        pytest.skip("the shared experts do not depend on the routed experts' activation path")
     torch.manual_seed(21)
     m = MoE(hidden_size=128, intermediate_size=64, shared_intermediate_size=shared, num_experts=8,
-            num_experts_per_tok=2, activation_function="swiglu", add_bias=False, dropout=0.0, init_method="normal",
+            num_experts_per_tok=2, activation_function=activation, add_bias=False, dropout=0.0, init_method="normal",
             initializer_range=0.1, m_width=None, num_layers=1, use_padding_free_transformer=True)
     m = m.to(dtype).to(device).train()
     x0 = torch.randn(300, 128, device=device, dtype=dtype)
