@@ -981,7 +981,24 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   // ---- epilogue of one tile: acc -> (SwiGLU) -> LDS scratch -> 16-byte row-contiguous stores -----------
   T* __restrict__ out = static_cast<T*>(a.out);
   static_assert(!PP || NW * EPI_BYTES <= STAGE_BYTES, "epilogue scratch must fit the free ring stage");
-  auto epilogue = [&](const TileCoord& tc) {
+  constexpr int RPP = 64 / EPI_CPR;  // rows per read-back pass
+  constexpr int MP = MB / EPI_MB;    // 32-row passes over the wave's token rows
+  // Destination rows of everything this lane will store in a tile's epilogue.  With scattered output they are
+  // fetched one tile ahead (next to the gather indices of the tile after), so that the epilogue does not start
+  // with a memory latency.
+  struct OutRows {
+    int r[MP][32 / RPP];
+  };
+  auto load_out_rows = [&](const TileCoord& tc, OutRows& o) {
+#pragma unroll
+    for (int mp = 0; mp < MP; ++mp)
+#pragma unroll
+      for (int it = 0; it < 32 / RPP; ++it) {
+        const int row = tc.row_begin + wm * WTM + mp * 32 + it * RPP + lane / EPI_CPR;
+        o.r[mp][it] = (a.scatter && row < tc.row_end) ? a.sorted_scattered[row] : row;
+      }
+  };
+  auto epilogue = [&](const TileCoord& tc, const OutRows& orows) {
     // PP: the ring stage consumed last is free until the next tile's first memory phase refills it (the
     // tile loop puts a barrier between this epilogue and that refill)
     unsigned char* scratch = PP ? smem_raw + ((g + NSTAGE - 1) & (NSTAGE - 1)) * STAGE_BYTES + wave * EPI_BYTES
@@ -989,18 +1006,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     // scratch row r keeps its EPI_CPR 16-byte chunks at slots chunk ^ swz(r): the 8-byte writes of a
     // wave and the 16-byte read-back both spread over all banks
     auto swz = [](int r) { return EPI_CPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3); };
-    constexpr int RPP = 64 / EPI_CPR;  // rows per read-back pass
-    constexpr int MP = MB / EPI_MB;    // 32-row passes over the wave's token rows
-    // destination rows of everything this lane will store, fetched up front: one memory latency per tile
-    // instead of one per store
-    int orow_of[MP][32 / RPP];
-#pragma unroll
-    for (int mp = 0; mp < MP; ++mp)
-#pragma unroll
-      for (int it = 0; it < 32 / RPP; ++it) {
-        const int row = tc.row_begin + wm * WTM + mp * 32 + it * RPP + lane / EPI_CPR;
-        orow_of[mp][it] = (a.scatter && row < tc.row_end) ? a.sorted_scattered[row] : row;
-      }
+    const auto& orow_of = orows.r;
 #pragma unroll
     for (int mp = 0; mp < MP; ++mp) {
 #pragma unroll
@@ -1069,8 +1075,10 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     load_rows(c1, raw1);
     make_src(c0, raw0, src_cur);
     make_src(c1, raw1, src_next);
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
   }
+  OutRows out_cur, out_next;
+  load_out_rows(c0, out_cur);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
   constexpr int AHEAD = PP ? NSTAGE - 1 : NSTAGE;  // slices in flight ahead of the one being consumed
   static_assert(!PP || (BK == 32 && WN == 2), "ping-pong shape");
 #pragma unroll
@@ -1101,7 +1109,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     if (t2 >= 0) locate(t2, c2);
     int raw2[NXLD];
     load_rows(c2, raw2);
-    epilogue(c0);
+    load_out_rows(c1, out_next);
+    epilogue(c0, out_cur);
     if (PP) {
       // every wave is done with its scratch before any wave's DMA of the next tile lands in that stage
       __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
@@ -1119,6 +1128,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     c1 = c2;
     t1 = t2;
     src_cur = src_next;
+    out_cur = out_next;
     make_src(c2, raw2, src_next);
     // Retire every load the compiler knows about (row indices, epilogue traffic) here, once per tile:
     // otherwise it re-checks them with vmcnt(0) inside the slice loop and drains the DMA ring there.
