@@ -17,8 +17,9 @@
 //   * An expert's rows are cut into groups of `chunk` rows; a work item is one 256 x 256 output tile of one
 //     group.  Items are dealt so that the 32 workgroups of an XCD work on the tiles of the same few groups at
 //     the same time: the group's rows are then fetched from HBM once per XCD and shared through its L2.
-//     Every item writes an fp32 partial tile; a second kernel sums the partials of an expert in group order
-//     and rounds once (deterministic, and experts without rows get zeros).
+//     An item of an expert with several groups writes an fp32 partial tile and a second kernel sums the partials
+//     of the expert in group order and rounds once (deterministic); an expert with one group is written directly,
+//     one without rows gets zeros from the second kernel.
 //   * HBM -> LDS by DMA (no registers), a ring of four 32-row slices with three in flight, and the forward
 //     kernel's ping-pong schedule: the two waves of a SIMD alternate between a memory phase and a matrix phase.
 //     A row's address is a scalar (index loads go through the scalar cache), the lanes add constant offsets.
@@ -51,6 +52,7 @@ struct WgradArgs {
   const int32_t* b_idx;           // same for `b`
   const int32_t* expert_offsets;  // (E,) inclusive ends of the experts' row ranges
   float* partial;                 // [group][M][N]
+  void* dw;                       // (E, M, N): written directly for an expert with a single group
   int* next_item;                 // [8] per-XCD work counters, zero on entry
   int L, M, N, E, chunk, m_tiles, n_tiles;
 };
@@ -193,11 +195,20 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
     __syncthreads();
     if (item >= items_x) break;
     const int grp = gbeg + item / tiles;
+    // A group's tiles are numbered in bands of 8 row tiles, column tile slowest inside a band: the 32 workgroups
+    // of the XCD, which hold 32 consecutive items, then cover 8 x 4 tiles -- 12 operand slabs for 32 tiles.  (Row
+    // tile fastest over all of them would re-read every A slab once per column tile: with 112 x 16 tiles that is
+    // 16 passes over the whole A operand.)
     const int tile = item % tiles;
-    const int mt = tile % a.m_tiles, nt = tile / a.m_tiles;
+    const int band = tile / (8 * a.n_tiles);
+    const int rem = tile - band * 8 * a.n_tiles;
+    const int left = a.m_tiles - band * 8;
+    const int width = left < 8 ? left : 8;
+    const int nt = rem / width;
+    const int mt = band * 8 + rem - nt * width;
 
     // group -> expert and its row range (wave-uniform)
-    int r0 = 0, r1 = 1;
+    int r0 = 0, r1 = 1, expert = 0, expert_groups = 1;
     for (int e0 = 0; e0 < a.E; e0 += 64) {
       const int e = e0 + lane;
       const int incl = e < a.E ? etab[2 * e] : 0x7fffffff;
@@ -206,6 +217,8 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
         const int ex = e0 + __ffsll((long long)hit) - 1;
         const int first = ex > 0 ? etab[2 * (ex - 1)] : 0;
         const int prev = ex > 0 ? etab[2 * (ex - 1) + 1] : 0;
+        expert = ex;
+        expert_groups = etab[2 * ex] - first;
         const int rows = group_rows(etab[2 * ex + 1] - prev, etab[2 * ex] - first);
         r0 = prev + (grp - first) * rows;
         r1 = etab[2 * ex + 1];
@@ -215,6 +228,8 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
     }
     r0 = __builtin_amdgcn_readfirstlane(r0);
     r1 = __builtin_amdgcn_readfirstlane(r1);
+    expert = __builtin_amdgcn_readfirstlane(expert);
+    expert_groups = __builtin_amdgcn_readfirstlane(expert_groups);
     const int nk = (r1 - r0 + BK - 1) / BK;
 
     // lane offsets of this tile; columns past the operand's width re-read the tile's first piece (their
@@ -329,21 +344,40 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
-    // ---- fp32 partial tile: register i of block (mb, nb) is row 16 mb + 4 (lane / 16) + i, column 16 nb + lane % 16
-    float* __restrict__ out = a.partial + (size_t)grp * a.M * a.N;
+    // ---- output tile: register i of block (mb, nb) is row 16 mb + 4 (lane / 16) + i, column 16 nb + lane % 16.
+    // An expert with one group is final: rounded and written straight into dw (whole 32-byte sectors per 16
+    // lanes).  Otherwise an fp32 partial tile for the reduction kernel.
+    if (expert_groups == 1) {
+      T* __restrict__ out = static_cast<T*>(a.dw) + (size_t)expert * a.M * a.N;
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+      for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int m = mt * TILE + wm * 64 + mb * 16 + 4 * fq + i;
-        if (m < a.M) {
+        for (int i = 0; i < 4; ++i) {
+          const int m = mt * TILE + wm * 64 + mb * 16 + 4 * fq + i;
+          if (m < a.M) {
 #pragma unroll
-          for (int nb = 0; nb < 8; ++nb) {
-            const int n = nt * TILE + wn * 128 + nb * 16 + fi;
-            if (n < a.N) out[(size_t)m * a.N + n] = acc[mb][nb][i];
+            for (int nb = 0; nb < 8; ++nb) {
+              const int n = nt * TILE + wn * 128 + nb * 16 + fi;
+              if (n < a.N) Elt<T>::store(out + (size_t)m * a.N + n, acc[mb][nb][i]);
+            }
           }
         }
-      }
+    } else {
+      float* __restrict__ out = a.partial + (size_t)grp * a.M * a.N;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int m = mt * TILE + wm * 64 + mb * 16 + 4 * fq + i;
+          if (m < a.M) {
+#pragma unroll
+            for (int nb = 0; nb < 8; ++nb) {
+              const int n = nt * TILE + wn * 128 + nb * 16 + fi;
+              if (n < a.N) out[(size_t)m * a.N + n] = acc[mb][nb][i];
+            }
+          }
+        }
+    }
   }
 }
 
@@ -351,7 +385,8 @@ __global__ void wgrad_zero_counters_kernel(int* counters) {
   if (threadIdx.x < 8) counters[threadIdx.x] = 0;
 }
 
-// dW[e] = sum of expert e's partial slabs in group order, rounded once; zeros for an expert without rows
+// dW[e] = sum of expert e's partial slabs in group order, rounded once (experts with several groups); zeros for an
+// expert without rows
 template <typename T>
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ partial,
                                                            const int32_t* __restrict__ offsets, T* __restrict__ dw,
@@ -364,6 +399,7 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restri
     prev = end;
   }
   const int count = (offsets[e] - prev + chunk - 1) / chunk;
+  if (count == 1) return;  // written by the main kernel
   const long n8 = mn / 8;
   for (long id = (long)blockIdx.x * 256 + threadIdx.x; id < n8; id += (long)gridDim.x * 256) {
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -420,6 +456,7 @@ extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const v
   WgradArgs g;
   g.a = a; g.b = b; g.a_idx = a_idx; g.b_idx = b_idx; g.expert_offsets = expert_offsets;
   g.partial = static_cast<float*>(workspace);
+  g.dw = dw;
   g.next_item = nullptr;
   g.L = L; g.M = M; g.N = N; g.E = E;
   g.chunk = wgrad_chunk(L, M, N);
