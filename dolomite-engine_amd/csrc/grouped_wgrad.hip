@@ -119,6 +119,8 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
   constexpr int NSTAGE = 4, AHEAD = 3;
   constexpr int NLD = 4;                   // DMA instructions per wave and slice (4 row pairs)
   typedef const __attribute__((address_space(4))) int32_t* const_idx_t;
+  typedef int32_t i32x8_a4 __attribute__((ext_vector_type(8), aligned(4)));
+  typedef const __attribute__((address_space(4))) i32x8_a4* const_idx8_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   int* etab = reinterpret_cast<int*>(smem_raw + NSTAGE * STAGE_BYTES);
   int* item_slot = etab + 2 * a.E;
@@ -166,7 +168,6 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
   const int wq = wave & 3;
   const unsigned char* src = static_cast<const unsigned char*>(load_b ? a.b : a.a);
   const const_idx_t idx = reinterpret_cast<const_idx_t>(reinterpret_cast<uintptr_t>(load_b ? a.b_idx : a.a_idx));
-  const bool gathered = idx != nullptr;
   const int ld = load_b ? a.N : a.M;  // columns of the operand
   const uint32_t ldbytes32 = (uint32_t)ld * (uint32_t)sizeof(T);  // operands stay below 4 GiB (checked on the host)
   // LDS position lane % 32 of row `krow` holds the logical 16-byte piece whose 32-byte group is
@@ -188,6 +189,9 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
 
   // Items of an XCD are handed out in order through a counter: the workgroups of the XCD stay on neighbouring
   // items (same group of rows, shared through the L2) and none of them idles while another still has a queue.
+  // (instantiated twice: for an operand gathered through an index array and for one read in place)
+  auto run_items = [&](auto gather_tag) {
+  constexpr bool GATHER = decltype(gather_tag)::value;
   for (;;) {
     if (tid == 0) *item_slot = atomicAdd(a.next_item + xcd, 1);
     __syncthreads();
@@ -243,11 +247,19 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
     // rows of slice `slice` this wave fetches: sorted rows r0 + 32 slice + 8 wq + [0, 8), clamped into the group
     // (rows past its end are fetched again from its last row and masked out of the last slice's fragments)
     auto load_idx = [&](int slice, int (&rw)[8]) {
+      const int first = r0 + slice * BK + 8 * wq;
+      if (GATHER && first + 7 < r1) {
+        // the usual case: eight consecutive indices in one scalar load
+        const i32x8_a4 v = *reinterpret_cast<const_idx8_t>(idx + first);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        int r = r0 + slice * BK + 8 * wq + i;
-        if (r > r1 - 1) r = r1 - 1;
-        rw[i] = gathered ? idx[r] : r;
+        for (int i = 0; i < 8; ++i) rw[i] = v[i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          int r = first + i;
+          if (r > r1 - 1) r = r1 - 1;
+          rw[i] = GATHER ? idx[r] : r;
+        }
       }
     };
     auto dma_slice = [&](const int (&rw)[8], int stage) {
@@ -321,9 +333,11 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
     if (wn == 1) __builtin_amdgcn_s_barrier();
     for (int g = 0; g < nk; ++g) {
       const int cur = g & (NSTAGE - 1), fill = (g + AHEAD) & (NSTAGE - 1);
-      read_frags(cur);
-      // slices past the group's end are fetched like the others (clamped rows) and never multiplied
+      // slices past the group's end are fetched like the others (clamped rows) and never multiplied.  The DMA goes
+      // first: its row indices came in long ago, and a wait for them behind the fragment reads would also wait
+      // for those (scalar loads and LDS reads share a counter)
       dma_slice(rw, fill);
+      read_frags(cur);
       if (g == nk - 1 && last_rows < BK) mask_frags();
       asm volatile("" ::: "memory");
       // own DMA of slice g + 1 has landed (g + 2 and g + 3 stay in flight); fragments are in registers
@@ -379,6 +393,9 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
         }
     }
   }
+  };
+  if (idx != nullptr) run_items(std::true_type{});
+  else run_items(std::false_type{});
 }
 
 __global__ void wgrad_zero_counters_kernel(int* counters) {
