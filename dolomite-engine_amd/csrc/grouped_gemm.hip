@@ -923,9 +923,9 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
 
   auto mfma_step = [&](int buf) {
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
+    for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
+      for (int nb = 0; nb < NB; ++nb) {
         if constexpr (PP) acc[nb][mb] = Mfma16<T>::run(wf[buf][nb], xf[buf][mb], acc[nb][mb]);
         else acc[nb][mb] = Mfma32<T>::run(wf[buf][nb], xf[buf][mb], acc[nb][mb]);
       }
