@@ -90,6 +90,22 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_fp8_tiled_bytes(64, 4096, 1408, 0) == 64 * 4096 * 1408
     assert lib.mi_moe_fp8_tiled_bytes(4, 20, 256, 1) == 4 * 2 * 2 * 4096  # 20 channels pad to two units
     assert lib.mi_moe_fp8_tiled_bytes(4, 20, 200, 1) == 0
+    # backward entry points
+    assert lib.mi_moe_scattered_gemm_wt(None, None, None, None, None, 16, 128, 8, 4, 2, 0, 1, _lib.F32, None) == E_NULL
+    assert lib.mi_moe_scattered_gemm_wt(None, None, None, None, None, 0, 128, 8, 4, 2, 0, 1, _lib.BF16, None) == 0
+    assert lib.mi_moe_grouped_wgrad(None, None, None, None, None, None, None, 0, 16, 16, 16, 12, 8, 4, _lib.BF16, None) == E_UNSUP
+    assert lib.mi_moe_grouped_wgrad(None, None, None, None, None, None, None, 0, 16, 16, 16, 8, 8, 300, _lib.BF16, None) == E_UNSUP
+    assert lib.mi_moe_grouped_wgrad(None, None, None, None, None, None, None, 0, 16, 16, 16, 8, 8, 4, _lib.F32, None) == E_DTYPE
+    assert lib.mi_moe_grouped_wgrad(None, None, None, None, None, None, None, 0, 16, 16, 16, 8, 8, 4, _lib.BF16, None) == E_NULL
+    assert lib.mi_moe_grouped_wgrad_workspace_bytes(262144, 40, 1024, 1536) > 0
+    assert lib.mi_moe_swiglu_backward(None, None, None, None, None, None, None, 4, 12, _lib.BF16, None) == E_UNSUP
+    assert lib.mi_moe_swiglu_backward(None, None, None, None, None, None, None, 4, 16, _lib.F32, None) == E_DTYPE
+    assert lib.mi_moe_swiglu_backward(None, None, None, None, None, None, None, 0, 16, _lib.BF16, None) == 0
+    assert lib.mi_moe_combine_grad_gates(None, None, None, 4, 2, 16, _lib.BF16, None) == E_NULL
+    assert lib.mi_moe_aux_loss(None, None, None, None, 0, 4, 300, 2, _lib.BF16, None) == E_UNSUP
+    assert lib.mi_moe_aux_loss(None, None, None, None, 0, 4, 8, 2, _lib.BF16, None) == E_NULL
+    assert lib.mi_moe_aux_loss_workspace_bytes(64, 8) == (2 + 1) * 17 * 4
+    assert lib.mi_moe_aux_loss_backward(None, None, None, None, 4, 8, _lib.BF16, None) == E_NULL
 
 
 def test_missing_library_fails_loudly(monkeypatch):
