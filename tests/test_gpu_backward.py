@@ -250,3 +250,38 @@ def test_scattered_experts_is_differentiable(device, dtype, mode, gated, T, E, k
     for name, got, want in (("x", xd.grad, xr.grad), ("w", wd.grad, wr.grad)) + ((("gates", gd.grad, gr.grad),) if gated else ()):
         scale = want.abs().max().clamp_min(1e-6)
         torch.testing.assert_close(got.cpu().float() / scale, want / scale, rtol=tol["rtol"], atol=tol["rtol"]), name
+
+
+def test_grouped_wgrad_full_size(device):
+    """Granite-3B-A800M-shape weight gradients (262144 sorted rows, 40 experts, Zipf-like sizes, both uses of the
+    kernel): every expert's block against a float32 product of the same rows computed by torch on the GPU, and the
+    sum over experts against one dense product (a checksum that every row was used exactly once)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(11)
+    T, k, E, H, I = 32768, 8, 40, 1536, 512
+    L = T * k
+    w = 1.0 / torch.arange(1, E + 1, dtype=torch.float64) ** 1.1
+    counts = torch.distributions.Multinomial(L, (w / w.sum()).float()).sample().long()
+    counts = counts[torch.randperm(E, generator=g)]
+    offsets = counts.cumsum(0).to(torch.int32).to(device)
+    tok = torch.randint(0, T, (L,), generator=g, dtype=torch.int32).to(device)
+    d_h = (torch.randn(L, 2 * I, generator=g) * 0.5).to(torch.bfloat16).to(device)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(device)
+
+    dw = ops.grouped_wgrad(d_h, x, offsets, None, tok)            # d c_fc: (E, 2I, H)
+    assert tuple(dw.shape) == (E, 2 * I, H)
+    xg = x[tok.long()]
+    dense = d_h.float().t() @ xg.float()
+    torch.testing.assert_close(dw.float().sum(0), dense, rtol=2e-2, atol=2e-2 * dense.abs().max().item())
+    start = 0
+    for e, end in enumerate(offsets.tolist()):
+        if e % 7 == 0 or counts[e] == counts.max():
+            ref = d_h[start:end].float().t() @ xg[start:end].float()
+            torch.testing.assert_close(dw[e].float(), ref, rtol=2e-2, atol=1e-2 * ref.abs().max().item())
+        start = end
+
+    dy = torch.randn(T, H, generator=g).to(torch.bfloat16).to(device)
+    act = (torch.randn(L, I, generator=g) * 0.5).to(torch.bfloat16).to(device)
+    dp = ops.grouped_wgrad(dy, act, offsets, tok, None)           # d c_proj: (E, H, I)
+    dense = dy[tok.long()].float().t() @ act.float()
+    torch.testing.assert_close(dp.float().sum(0), dense, rtol=2e-2, atol=2e-2 * dense.abs().max().item())
