@@ -285,3 +285,26 @@ def test_grouped_wgrad_full_size(device):
     dp = ops.grouped_wgrad(dy, act, offsets, tok, None)           # d c_proj: (E, H, I)
     dense = dy[tok.long()].float().t() @ act.float()
     torch.testing.assert_close(dp.float().sum(0), dense, rtol=2e-2, atol=2e-2 * dense.abs().max().item())
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_grouped_wgrad_random_shapes(device, seed):
+    """Random shapes around the kernel's boundaries: row counts that straddle the group size, operand widths that
+    leave partial 256-column tiles or more than 8 row tiles (several bands), many experts."""
+    import random
+
+    rnd = random.Random(seed)
+    E = rnd.choice([1, 2, 7, 33, 64, 200, 256])
+    L = rnd.choice([1, 31, 255, 257, 1000, 4097, 9001])
+    M = 8 * rnd.choice([1, 5, 32, 33, 40, 260, 300])
+    N = 8 * rnd.choice([1, 3, 31, 32, 65])
+    g = torch.Generator().manual_seed(seed)
+    counts = torch.distributions.Multinomial(L, torch.rand(E, generator=g).pow(4) + 1e-6).sample().long()
+    offsets = counts.cumsum(0).to(torch.int32)
+    rows_other = rnd.choice([1, 17, L])
+    a = torch.randn(L, M, generator=g).to(torch.bfloat16)
+    b = torch.randn(rows_other, N, generator=g).to(torch.bfloat16)
+    b_idx = torch.randint(0, rows_other, (L,), generator=g, dtype=torch.int32)
+    got = _ops().grouped_wgrad(a.to(device), b.to(device), offsets.to(device), None, b_idx.to(device))
+    ref = _wgrad_reference(a, b, offsets, None, b_idx)
+    torch.testing.assert_close(got.cpu().double(), ref, rtol=2.0 ** -7, atol=2e-5 * max(1.0, counts.max().item()) ** 0.5 + 1e-6)
