@@ -35,6 +35,7 @@ SIGNATURES: dict[str, tuple] = {
     "mi_moe_count": (_i, [_vp, _i, _i, _vp, _vp]),
     "mi_moe_sort_bin_workspace_bytes": (_sz, [_i, _i]),
     "mi_moe_sort_bin": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "mi_moe_sort_bin_static": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "mi_moe_scattered_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mi_moe_scattered_gemm_wt": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mi_moe_scattered_gemm_cfg": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
@@ -57,6 +58,7 @@ SIGNATURES: dict[str, tuple] = {
 # return codes of include/mi_moe.h that callers branch on
 MI_MOE_EDTYPE = -3
 MI_MOE_EUNSUPPORTED = -6
+MI_MOE_ETOOLARGE = -7
 
 _lib = None
 _lock = threading.Lock()

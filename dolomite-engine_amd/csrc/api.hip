@@ -12,6 +12,7 @@ extern "C" const char* mi_moe_strerror(int rc) {
     case MI_MOE_EALIGN: return "mi_moe: a pointer or leading dimension is not aligned as required";
     case MI_MOE_EWORKSPACE: return "mi_moe: workspace missing or too small";
     case MI_MOE_EUNSUPPORTED: return "mi_moe: shape / option combination not supported by this entry point";
+    case MI_MOE_ETOOLARGE: return "mi_moe: input needs more scratch memory than this non-allocating entry point holds";
     default: break;
   }
   if (rc > 0) return hipGetErrorString(static_cast<hipError_t>(rc));

@@ -405,3 +405,61 @@ extern "C" int mi_moe_sort_bin(const int32_t* topk_idx, int T, int k, int E, int
                      sorted_expert, sorted_scattered);
   return mi_launch_status();
 }
+
+// ------------------------------------------------------------------------------------------------
+// mi_moe_sort_bin with its workspace inside the library: for callers that cannot allocate.
+// ------------------------------------------------------------------------------------------------
+//
+// The chunk histograms and expert bases of the three-pass sort live in a fixed array in device memory instead of a
+// caller workspace.  The array's name is only a handle on the host: the address the kernels get comes from
+// hipGetSymbolAddress, asked once per device (each device holds its own copy at its own address) the first time the
+// entry point runs with that device current.  Nothing in the array has to start at zero: every word pass 2 and
+// pass 3 read was written by pass 1 / pass 2 of the same call.  Calls that overlap on one device share the array and
+// race.
+
+#include <mutex>
+
+#define SORT_STATIC_BYTES MI_MOE_SORT_BIN_STATIC_BYTES
+#define SORT_STATIC_MAX_DEVICES 64
+
+static __device__ __align__(256) unsigned char scratch[SORT_STATIC_BYTES];
+
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[SORT_STATIC_MAX_DEVICES];  // written once per device under the mutex, read-only afterwards
+
+// Device address of `scratch` on the current device (0 with *rc set on failure).
+static int32_t* sort_static_scratch(int* rc) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { *rc = (int)e; return nullptr; }
+  if (dev < 0 || dev >= SORT_STATIC_MAX_DEVICES) { *rc = MI_MOE_EUNSUPPORTED; return nullptr; }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) { *rc = (int)e; return nullptr; }
+    if (!p || !mi_aligned(p, 16)) { *rc = MI_MOE_EALIGN; return nullptr; }
+    g_scratch_ptr[dev] = p;
+  }
+  *rc = MI_MOE_OK;
+  return static_cast<int32_t*>(g_scratch_ptr[dev]);
+}
+
+extern "C" int mi_moe_sort_bin_static(const int32_t* topk_idx, int T, int k, int E, int32_t* sorted_expert,
+                                      int32_t* sorted_scattered, int32_t* expert_offsets, mi_moe_stream_t stream) {
+  if (T < 0 || k < 1 || E < 1 || E > SORT_MAX_E) return MI_MOE_ESHAPE;
+  if ((int64_t)T * k > (int64_t)0x7fffffff - SORT_CHUNK) return MI_MOE_ESHAPE;
+  if (!expert_offsets) return MI_MOE_ENULL;
+  const int L = T * k;
+  if (L > 0 && (!topk_idx || !sorted_expert || !sorted_scattered)) return MI_MOE_ENULL;
+  const size_t need = mi_moe_sort_bin_workspace_bytes(L, E);
+  if (need > SORT_STATIC_BYTES) return MI_MOE_ETOOLARGE;
+  int32_t* ws = nullptr;
+  if (need) {
+    int rc = MI_MOE_OK;
+    ws = sort_static_scratch(&rc);
+    if (!ws) return rc;
+  }
+  // the one-block path (need == 0) touches no workspace; otherwise the same three launches on the library's array
+  return mi_moe_sort_bin(topk_idx, T, k, E, sorted_expert, sorted_scattered, expert_offsets, ws, need, stream);
+}

@@ -3,14 +3,16 @@
  *
  * One shared library (libmi_moe.so), plain C types only.  Every function
  *   - takes device pointers the CALLER allocated (inputs, outputs and workspace); the library
- *     never allocates, frees or keeps a pointer after it returns;
+ *     never allocates, frees or keeps a pointer after it returns (mi_moe_sort_bin_static, which brings
+ *     its own fixed scratch array, is the one documented exception to "workspace");
  *   - validates its arguments on the host BEFORE anything is launched and returns
  *       0  on success,
  *      <0  an MI_MOE_E* argument / shape / alignment / dtype error (nothing was launched),
  *      >0  the hipError_t of a failed launch;
  *   - is asynchronous: work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
  *     default stream); there is no host synchronisation and no device-to-host copy;
- *   - is re-entrant and keeps no mutable global state.
+ *   - is re-entrant and keeps no mutable global state (values the library reads once and then only
+ *     reads back -- device attributes, the address of that scratch array -- are cached per device).
  *
  * Index tensors are int32 inside the ABI.  Matrices are row-major and contiguous.  Expert weights
  * are read in the module's native (E, out_features, in_features) layout, i.e. the contraction
@@ -45,6 +47,7 @@ extern "C" {
 #define MI_MOE_EALIGN (-4)     /* a pointer or leading dimension is not aligned as required */
 #define MI_MOE_EWORKSPACE (-5) /* workspace missing or too small */
 #define MI_MOE_EUNSUPPORTED (-6)
+#define MI_MOE_ETOOLARGE (-7)  /* input needs more scratch than a non-allocating entry point holds */
 
 typedef void* mi_moe_stream_t; /* hipStream_t */
 
@@ -116,6 +119,22 @@ size_t mi_moe_sort_bin_workspace_bytes(int L, int E);
 int mi_moe_sort_bin(const int32_t* topk_idx, int T, int k, int E, int32_t* sorted_expert,
                     int32_t* sorted_scattered, int32_t* expert_offsets, void* ws, size_t ws_bytes,
                     mi_moe_stream_t stream);
+
+/*
+ * mi_moe_sort_bin without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same inputs, outputs and results as mi_moe_sort_bin; the chunk histograms live in a fixed array of
+ * MI_MOE_SORT_BIN_STATIC_BYTES that the library keeps in device memory on every GPU it runs on (held until the
+ * process ends).  Inputs that need more -- mi_moe_sort_bin_workspace_bytes(T*k, E) > MI_MOE_SORT_BIN_STATIC_BYTES,
+ * e.g. more than about 2^18 / E * 2048 slots -- are refused with MI_MOE_ETOOLARGE before anything is launched.
+ * Calls no hipMalloc / hipFree; the first call on a device looks the array's address up (hipGetSymbolAddress) and
+ * keeps it, which is the only state the library holds (make that first call outside graph capture).  All calls on
+ * one GPU share the array: calls that overlap on one GPU (different streams or host threads) race; calls on one
+ * stream are ordered and safe.
+ */
+#define MI_MOE_SORT_BIN_STATIC_BYTES (1u << 20)
+int mi_moe_sort_bin_static(const int32_t* topk_idx, int T, int k, int E, int32_t* sorted_expert,
+                           int32_t* sorted_scattered, int32_t* expert_offsets, mi_moe_stream_t stream);
 
 /*
  * Grouped ("scatter2scatter") GEMM:  for every sorted row i with expert e_i

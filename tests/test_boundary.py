@@ -55,7 +55,7 @@ def test_abi_version_and_error_text():
     header = open(HEADER).read()
     assert f"#define MI_MOE_ABI_VERSION {_lib.ABI_VERSION}" in header
     for code, word in [(0, "ok"), (-1, "NULL"), (-2, "dimension"), (-3, "element type"), (-4, "aligned"),
-                       (-5, "workspace"), (-6, "not supported")]:
+                       (-5, "workspace"), (-6, "not supported"), (-7, "scratch")]:
         assert word in lib.mi_moe_strerror(code).decode()
     assert "unknown" in lib.mi_moe_strerror(-99).decode()
 
@@ -77,6 +77,12 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_sort_bin(None, 4, 2, 8, None, None, None, None, 0, None) == E_NULL
     assert lib.mi_moe_sort_bin_workspace_bytes(1000, 8) == 0  # small inputs need no workspace
     assert lib.mi_moe_sort_bin_workspace_bytes(262144, 40) == (40 * 128 + 40) * 4
+    # the non-allocating variant: same checks, and inputs beyond its fixed scratch array are refused on the host
+    assert lib.mi_moe_sort_bin_static(None, 4, 2, 0, None, None, None, None) == E_SHAPE
+    assert lib.mi_moe_sort_bin_static(None, 4, 2, 8, None, None, None, None) == E_NULL
+    assert lib.mi_moe_sort_bin_workspace_bytes(1 << 23, 1000) > (1 << 20)
+    assert lib.mi_moe_sort_bin_static(ctypes.c_void_p(256), 1 << 20, 8, 1000, ctypes.c_void_p(256), ctypes.c_void_p(256),
+                                      ctypes.c_void_p(256), None) == -7
     assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 16, 0, 8, 4, 2, 0, 1, _lib.BF16, None) == E_SHAPE
     assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 16, 8, 8, 4, 2, 0, 1, 7, None) == E_DTYPE
     assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 16, 8, 8, 4, 2, 0, 1, _lib.BF16, None) == E_NULL
