@@ -47,6 +47,7 @@ SIGNATURES: dict[str, tuple] = {
     "mi_moe_combine_grad_gates": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mi_moe_grouped_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mi_moe_grouped_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "mi_moe_grouped_wgrad_naive": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "mi_moe_aux_loss_workspace_bytes": (_sz, [_i, _i]),
     "mi_moe_aux_loss": (_i, [_vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "mi_moe_aux_loss_backward": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -57,6 +58,7 @@ SIGNATURES: dict[str, tuple] = {
 
 # return codes of include/mi_moe.h that callers branch on
 MI_MOE_EDTYPE = -3
+MI_MOE_EALIGN = -4
 MI_MOE_EUNSUPPORTED = -6
 MI_MOE_ETOOLARGE = -7
 

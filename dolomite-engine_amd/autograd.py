@@ -4,7 +4,7 @@ The forward is the same three launches as in inference (up-projection with fused
 combine).  The backward reuses the grouped GEMM for everything that is a "rows times expert weight" product --
 the gradient w.r.t. the activations of both projections and the recomputation of the two intermediates that
 are not kept -- and a second kernel, a grouped X^T dY contracted over each expert's rows, for the weight
-gradients (fp32 and odd shapes fall back to one library GEMM per expert).  The reference gets both from the external scattermoe autograd function
+gradients (fp32 and odd shapes run a one-thread-per-element form of it; nothing synchronises with the host).  The reference gets both from the external scattermoe autograd function
 (lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:91-101); this module is the counterpart for the
 gradient, built on this package's forward kernels.
 
@@ -72,21 +72,8 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
 
         # weight gradients: per expert X^T dY over that expert's rows
         tok32 = torch.div(ss, k, rounding_mode="floor").to(torch.int32)
-        if half and ops.grouped_wgrad_supported(d_h, x, E):
-            d_w_fc = ops.grouped_wgrad(d_h, x, off, None, tok32)
-            d_w_proj = ops.grouped_wgrad(dy, act_g, off, tok32, None)
-        else:
-            tok = tok32.long()
-            d_w_fc = torch.zeros_like(w_fc)
-            d_w_proj = torch.zeros_like(w_proj)
-            start = 0
-            for e, end in enumerate(off.tolist()):
-                if end > start:
-                    rows = slice(start, end)
-                    t_e = tok[rows]
-                    d_w_fc[e] = d_h[rows].t() @ x[t_e]
-                    d_w_proj[e] = dy[t_e].t() @ act_g[rows]
-                start = end
+        d_w_fc = ops.grouped_wgrad(d_h, x, off, None, tok32)
+        d_w_proj = ops.grouped_wgrad(dy, act_g, off, tok32, None)
         return dx, d_w_fc, d_w_proj, d_gates, None, None, None
 
 
@@ -100,7 +87,7 @@ class ScatteredExperts(torch.autograd.Function):
         with gates (T, kg):  y[t] = sum_j gates[t, j] * out[t * kg + j]
 
     Backward: d x from the transposed-weight form of the same kernel, d w from the grouped weight-gradient kernel
-    (16-bit dtypes; otherwise one library GEMM per expert), d gates from the recomputed rows."""
+    (matrix cores for 16-bit dtypes, a one-thread-per-element kernel otherwise), d gates from the recomputed rows."""
 
     @staticmethod
     def forward(ctx, x, w, k, sorted_scattered, expert_offsets, gates, grouped_in, grouped_out):
@@ -144,21 +131,9 @@ class ScatteredExperts(torch.autograd.Function):
 
         dw = None
         if need_w:
-            ssl = ss.long()
             a_idx = None if grouped_out else ss.to(torch.int32)
             b_idx = None if grouped_in else torch.div(ss, k, rounding_mode="floor").to(torch.int32)
-            if half and ops.grouped_wgrad_supported(d_out, x, E):
-                dw = ops.grouped_wgrad(d_out, x, off, a_idx, b_idx)
-            else:
-                dw = torch.zeros_like(w)
-                start = 0
-                for e, end in enumerate(off.tolist()):
-                    if end > start:
-                        rows = torch.arange(start, end, device=x.device)
-                        a = d_out[rows if a_idx is None else ssl[rows]]
-                        b = x[rows if b_idx is None else torch.div(ssl[rows], k, rounding_mode="floor")]
-                        dw[e] = a.t() @ b
-                    start = end
+            dw = ops.grouped_wgrad(d_out, x, off, a_idx, b_idx)
         return dx, dw, None, None, None, d_gates, None, None
 
 

@@ -84,6 +84,49 @@ static inline int mi_launch_status() {
   return e == hipSuccess ? MI_MOE_OK : (int)e;
 }
 
+// ---- per-device values that are read once and only read back afterwards ----------------------------------
+// The launch paths need the number of compute units and, per kernel, a one-time opt-in to more than 64 KiB of
+// dynamic LDS.  Both are properties of (device, kernel) that never change, so they are asked once per device and
+// cached: a launch then costs hipGetDevice (thread-local) plus the launch itself.
+
+#include <atomic>
+
+#define MI_MAX_DEVICES 64
+
+// number of compute units of the current device; *dev_out (optional) receives the device index
+static inline int mi_cu_count(int* cus, int* dev_out = nullptr) {
+  static std::atomic<int> cache[MI_MAX_DEVICES];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev_out) *dev_out = dev;
+  int c = (dev >= 0 && dev < MI_MAX_DEVICES) ? cache[dev].load(std::memory_order_relaxed) : 0;
+  if (c == 0) {
+    e = hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev >= 0 && dev < MI_MAX_DEVICES) cache[dev].store(c, std::memory_order_relaxed);
+  }
+  *cus = c;
+  return MI_MOE_OK;
+}
+
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per (kernel, device).  `done` is a per-kernel bit mask of the
+// devices already set up (callers keep one static mask per kernel instantiation).  The value asked for is the
+// kernel's upper bound, so a later launch with less LDS needs no second call.
+static inline int mi_allow_lds_once(const void* kern, int max_lds_bytes, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  const uint64_t bit = (dev >= 0 && dev < 64) ? (1ull << dev) : 0ull;
+  if (bit && (done.load(std::memory_order_acquire) & bit)) return MI_MOE_OK;
+  e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds_bytes);
+  if (e != hipSuccess) return (int)e;
+  if (bit) done.fetch_or(bit, std::memory_order_release);
+  return MI_MOE_OK;
+}
+
+#define MI_LDS_MAX_BYTES (160 * 1024)
+
 static inline bool mi_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 static inline int mi_ceil_div(int a, int b) { return (a + b - 1) / b; }

@@ -391,9 +391,9 @@ static int launch_decode_stream(DecodeArgs a, hipStream_t s) {
   const int lds = waves * DEC_WAVE_LDS;
   auto kern = a.tiled ? decode_fp8_stream_kernel<T, GLU, true> : decode_fp8_stream_kernel<T, GLU, false>;
   if (lds > 64 * 1024) {
-    hipError_t e =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return (int)e;
+    static std::atomic<uint64_t> lds_ok[2];  // one mask per kernel of this instantiation (tiled / row-major)
+    const int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), lds, lds_ok[a.tiled ? 1 : 0]);
+    if (rc != MI_MOE_OK) return rc;
   }
   const long grid = (units + waves - 1) / waves;
   if (grid > 0x7fffffffL) return MI_MOE_ESHAPE;

@@ -1169,9 +1169,9 @@ static int launch_tiled_k(GemmArgs a, hipStream_t s) {
   constexpr size_t lds = 2ull * (BM + BNW) * 64 * sizeof(T);
   auto kern = grouped_gemm_kernel<T, BM, BNW, WM, WN, GLU, KTAIL>;
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
+    static std::atomic<uint64_t> lds_ok{0};
+    const int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), (int)lds, lds_ok);
+    if (rc != MI_MOE_OK) return rc;
   }
   a.n_tiles = mi_ceil_div(a.N, BN);
   long max_m = (long)a.L / BM + (a.E < a.L ? a.E : a.L);
@@ -1194,9 +1194,9 @@ static int launch_dma(GemmArgs a, hipStream_t s) {
   constexpr size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T);
   auto kern = grouped_gemm_dma_kernel<T, BM, BNW, WM, WN, GLU>;
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
+    static std::atomic<uint64_t> lds_ok{0};
+    const int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), (int)lds, lds_ok);
+    if (rc != MI_MOE_OK) return rc;
   }
   a.n_tiles = mi_ceil_div(a.N, BN);
   long max_m = (long)a.L / BM + (a.E < a.L ? a.E : a.L);
@@ -1213,13 +1213,12 @@ static int launch_persistent(GemmArgs a, hipStream_t s) {
   constexpr int NW = WM * WN;
   const size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T) + (PP ? 0 : (size_t)NW * (NW > 4 ? 2048 : 4096)) + (size_t)a.E * 8;
   auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, BK, PP, WT>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) return (int)e;
+  static std::atomic<uint64_t> lds_ok{0};  // the expert table makes lds vary with E: opt in to the most it can be
+  int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok);
+  if (rc != MI_MOE_OK) return rc;
   a.n_tiles = mi_ceil_div(a.N, BN);
-  int dev = 0, cus = 0;
-  if ((e = hipGetDevice(&dev)) != hipSuccess) return (int)e;
-  if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return (int)e;
+  int cus = 0;
+  if ((rc = mi_cu_count(&cus)) != MI_MOE_OK) return rc;
   long max_tiles = ((long)a.L / BM + (a.E < a.L ? a.E : a.L)) * a.n_tiles;
   long grid = cus < max_tiles ? cus : max_tiles;
   grid = (grid + 7) / 8 * 8;
@@ -1261,13 +1260,16 @@ static int dispatch_cfg(GemmArgs a, int cfg, hipStream_t s) {
   }
 }
 
-static bool tiled_ok(const GemmArgs& a, int in_rows_bound, bool glu) {
+// Shapes the matrix-core kernels take: 16-byte chunks along K, 8-byte output pieces, 32-bit element offsets inside
+// one operand.
+static bool tiled_shape_ok(const GemmArgs& a, int in_rows_bound, bool glu) {
   if (a.K % 8 != 0 || a.N % 4 != 0) return false;
-  if (!mi_aligned(a.in, 16) || !mi_aligned(a.w, 16) || !mi_aligned(a.out, 8)) return false;
-  // 32-bit element offsets inside one operand
   if ((double)in_rows_bound * a.K >= 2147483648.0) return false;
   if ((double)(glu ? 2 : 1) * a.N * a.K >= 2147483648.0) return false;
   return true;
+}
+static bool tiled_aligned(const GemmArgs& a) {
+  return mi_aligned(a.in, 16) && mi_aligned(a.w, 16) && mi_aligned(a.out, 8);
 }
 
 static int pick_cfg(const GemmArgs& a) {
@@ -1278,10 +1280,14 @@ static int pick_cfg(const GemmArgs& a) {
   return 2;
 }
 
+// cfg < 0 picks a matrix-core kernel from the shape.  Nothing drops to the one-thread-per-output kernel on its own:
+// a 16-bit problem the matrix-core kernels cannot take is refused (MI_MOE_EALIGN for a misaligned pointer,
+// MI_MOE_EUNSUPPORTED for the shape) and the caller asks for cfg 3 explicitly if it wants the slow kernel.  fp32 has
+// no other kernel, so it takes cfg < 0 and cfg 3 alike.
 static int run_gemm(GemmArgs a, int dtype, bool glu, int cfg, int in_rows_bound, hipStream_t s) {
   if (a.L == 0) return MI_MOE_OK;
-  const bool fast = (dtype == MI_MOE_BF16 || dtype == MI_MOE_F16) && tiled_ok(a, in_rows_bound, glu);
-  if (cfg == 3 || !fast) {
+  const bool half = dtype == MI_MOE_BF16 || dtype == MI_MOE_F16;
+  if (cfg == 3 || !half) {
     if (cfg >= 0 && cfg != 3) return MI_MOE_EUNSUPPORTED;
     switch (dtype) {
       case MI_MOE_F32: return glu ? launch_naive<float, true>(a, s) : launch_naive<float, false>(a, s);
@@ -1290,6 +1296,8 @@ static int run_gemm(GemmArgs a, int dtype, bool glu, int cfg, int in_rows_bound,
       default: return MI_MOE_EDTYPE;
     }
   }
+  if (!tiled_shape_ok(a, in_rows_bound, glu)) return MI_MOE_EUNSUPPORTED;
+  if (!tiled_aligned(a)) return MI_MOE_EALIGN;
   if (cfg < 0) cfg = pick_cfg(a);
   if (dtype == MI_MOE_BF16) return glu ? dispatch_cfg<bf16_t, true>(a, cfg, s) : dispatch_cfg<bf16_t, false>(a, cfg, s);
   return glu ? dispatch_cfg<f16_t, true>(a, cfg, s) : dispatch_cfg<f16_t, false>(a, cfg, s);
@@ -1333,7 +1341,8 @@ extern "C" int mi_moe_scattered_gemm_wt(const void* in, const void* w_kn, void* 
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = K; a.N = N; a.E = E; a.kdiv = k; a.n_tiles = 0;
   a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1;
-  if (!tiled_ok(a, L, false) || !persistent_ok(a)) return MI_MOE_EUNSUPPORTED;
+  if (!tiled_shape_ok(a, L, false) || !persistent_ok(a)) return MI_MOE_EUNSUPPORTED;
+  if (!tiled_aligned(a)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == MI_MOE_BF16) return launch_persistent<bf16_t, 256, 256, 4, 2, false, 32, true, true>(a, s);
   return launch_persistent<f16_t, 256, 256, 4, 2, false, 32, true, true>(a, s);

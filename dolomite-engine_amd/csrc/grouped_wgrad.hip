@@ -485,10 +485,9 @@ extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const v
   g.m_tiles = mi_ceil_div(M, 256);
   g.n_tiles = mi_ceil_div(N, 256);
   const size_t lds = 4 * 2 * 32 * 256 * 2 + (size_t)E * 8 + 16;
-  int dev = 0, cus = 0;
-  hipError_t e;
-  if ((e = hipGetDevice(&dev)) != hipSuccess) return (int)e;
-  if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return (int)e;
+  int cus = 0;
+  int rc = mi_cu_count(&cus);
+  if (rc != MI_MOE_OK) return rc;
   const long max_items = wgrad_max_groups(L, E, g.chunk) * g.m_tiles * g.n_tiles;
   long grid = cus < max_items ? cus : max_items;
   grid = (grid + 7) / 8 * 8;
@@ -496,18 +495,66 @@ extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const v
   if (rblocks > 4096) rblocks = 4096;
   if (dtype == MI_MOE_BF16) {
     auto kern = grouped_wgrad_kernel<bf16_t>;
-    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess)
-      return (int)e;
+    static std::atomic<uint64_t> lds_ok{0};
+    if ((rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok)) != MI_MOE_OK) return rc;
     if (L > 0) hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, s, g);
     hipLaunchKernelGGL((wgrad_reduce_kernel<bf16_t>), dim3((unsigned)rblocks, (unsigned)E), dim3(256), 0, s, g.partial,
                        expert_offsets, static_cast<bf16_t*>(dw), E, mn, g.chunk);
   } else {
     auto kern = grouped_wgrad_kernel<f16_t>;
-    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess)
-      return (int)e;
+    static std::atomic<uint64_t> lds_ok{0};
+    if ((rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok)) != MI_MOE_OK) return rc;
     if (L > 0) hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, s, g);
     hipLaunchKernelGGL((wgrad_reduce_kernel<f16_t>), dim3((unsigned)rblocks, (unsigned)E), dim3(256), 0, s, g.partial,
                        expert_offsets, static_cast<f16_t*>(dw), E, mn, g.chunk);
+  }
+  return mi_launch_status();
+}
+
+// ---- any-shape / any-dtype weight gradient (one thread per element of dW) ------------------------------------
+// For fp32 and for shapes the matrix-core kernel above does not take.  Every element sums its expert's rows in
+// ascending order in fp32 (deterministic) and is rounded once.  Correct, not fast; no workspace, no host round trip.
+template <typename T>
+__global__ __launch_bounds__(256) void grouped_wgrad_naive_kernel(const T* __restrict__ a, const int32_t* __restrict__ a_idx,
+                                                                  const T* __restrict__ b, const int32_t* __restrict__ b_idx,
+                                                                  const int32_t* __restrict__ offsets, T* __restrict__ dw,
+                                                                  int M, int N) {
+  const int e = blockIdx.z;
+  const int n = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int m = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (m >= M || n >= N) return;
+  const int begin = e > 0 ? offsets[e - 1] : 0, end = offsets[e];
+  float acc = 0.f;
+  for (int r = begin; r < end; ++r) {
+    const size_t ar = a_idx ? (size_t)a_idx[r] : (size_t)r;
+    const size_t br = b_idx ? (size_t)b_idx[r] : (size_t)r;
+    acc = fmaf(Elt<T>::load(a + ar * M + m), Elt<T>::load(b + br * N + n), acc);
+  }
+  Elt<T>::store(dw + ((size_t)e * M + m) * N + n, acc);
+}
+
+extern "C" int mi_moe_grouped_wgrad_naive(const void* a, const int32_t* a_idx, const void* b, const int32_t* b_idx,
+                                          const int32_t* expert_offsets, void* dw, int L, int M, int N, int E, int dtype,
+                                          mi_moe_stream_t stream) {
+  if (L < 0 || M < 1 || N < 1 || E < 1 || E > 65535) return MI_MOE_ESHAPE;
+  if (dtype != MI_MOE_F32 && dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (!dw || !expert_offsets) return MI_MOE_ENULL;
+  if (L > 0 && (!a || !b)) return MI_MOE_ENULL;
+  const dim3 grid(mi_ceil_div(N, 64), mi_ceil_div(M, 4), E);
+  if (grid.y > 65535u) return MI_MOE_ESHAPE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case MI_MOE_F32:
+      hipLaunchKernelGGL((grouped_wgrad_naive_kernel<float>), grid, dim3(256), 0, s, static_cast<const float*>(a), a_idx,
+                         static_cast<const float*>(b), b_idx, expert_offsets, static_cast<float*>(dw), M, N);
+      break;
+    case MI_MOE_F16:
+      hipLaunchKernelGGL((grouped_wgrad_naive_kernel<f16_t>), grid, dim3(256), 0, s, static_cast<const f16_t*>(a), a_idx,
+                         static_cast<const f16_t*>(b), b_idx, expert_offsets, static_cast<f16_t*>(dw), M, N);
+      break;
+    default:
+      hipLaunchKernelGGL((grouped_wgrad_naive_kernel<bf16_t>), grid, dim3(256), 0, s, static_cast<const bf16_t*>(a), a_idx,
+                         static_cast<const bf16_t*>(b), b_idx, expert_offsets, static_cast<bf16_t*>(dw), M, N);
   }
   return mi_launch_status();
 }

@@ -576,17 +576,17 @@ static int launch_router_splitk(const void* x, const void* gw, const float* bias
 template <typename T, bool NORM>
 static int launch_router_lds(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
                              void* logits_out, void* gates, int32_t* idx, RouterNorm norm, size_t lds, hipStream_t s) {
-  int dev = 0, cus = 0;
-  hipError_t e;
-  if ((e = hipGetDevice(&dev)) != hipSuccess) return (int)e;
-  if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return (int)e;
+  int cus = 0;
+  int rc = mi_cu_count(&cus);
+  if (rc != MI_MOE_OK) return rc;
   const int groups = mi_ceil_div(T_, 16);
   const int blocks = groups < cus ? groups : cus;
   int waves = mi_ceil_div(groups, blocks);
   if (waves > ROUTER_LDS_WAVES) waves = ROUTER_LDS_WAVES;
   auto kern = waves > 4 ? router_fused_lds_kernel<T, 3, NORM> : router_fused_lds_kernel<T, 6, NORM>;
-  e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) return (int)e;
+  static std::atomic<uint64_t> lds_ok[2];  // the LDS size varies with E and H: opt in to the most it can be
+  rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok[waves > 4 ? 1 : 0]);
+  if (rc != MI_MOE_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(waves * 64), lds, s, static_cast<const T*>(x),
                      static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out),
                      static_cast<T*>(gates), idx, norm);

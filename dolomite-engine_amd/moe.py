@@ -323,8 +323,16 @@ class MoE(nn.Module):
         if self.router_logit_bias is not None:
             router_logits = (router_logits.float() + self.router_logit_bias.float()).to(router_logits.dtype)
 
-        if is_kernel_allowed(Kernel.scattermoe) and hidden_states.is_cuda and not torch.is_grad_enabled():
-            router_weights, selected_experts = ops.router_topk_softmax(router_logits, self.top_k)
+        if is_kernel_allowed(Kernel.scattermoe) and hidden_states.is_cuda:
+            # the kernel's tie rule (value descending, expert index ascending) in training and in inference alike:
+            # torch.topk documents no tie order, and bf16 logits tie often
+            with torch.no_grad():
+                router_weights, selected_experts = ops.router_topk_softmax(router_logits.detach(), self.top_k)
+            if torch.is_grad_enabled() and router_logits.requires_grad:
+                # the gradient flows through the selected logits: gather them at the kernel's indices and redo the
+                # softmax over the k values in torch (same arithmetic: fp32 softmax, one rounding)
+                picked = router_logits.gather(-1, selected_experts.long())
+                router_weights = F.softmax(picked.float(), dim=-1).type_as(hidden_states)
         else:
             router_weights, selected_experts = self._get_topk(router_logits)
             router_weights = F.softmax(router_weights.float(), dim=-1)

@@ -22,6 +22,16 @@ _DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
 
 _TIMER = None
+_WARNED: set = set()
+
+
+def _warn_once(key: str, message: str) -> None:
+    """Slow paths are taken loudly: one warning per process and kind."""
+    if key not in _WARNED:
+        _WARNED.add(key)
+        import warnings
+
+        warnings.warn(message, RuntimeWarning, stacklevel=3)
 
 
 def set_stage_timer(timer) -> None:
@@ -258,14 +268,31 @@ def scattered_gemm(inputs: torch.Tensor, weight: torch.Tensor, k: int, sorted_sc
                                               int(grouped_in), int(grouped_out), _code(inputs.dtype), _stream())
         if rc == 0:
             return out
-        if rc not in (_lib.MI_MOE_EUNSUPPORTED, _lib.MI_MOE_EDTYPE):
+        if rc not in (_lib.MI_MOE_EUNSUPPORTED, _lib.MI_MOE_EDTYPE, _lib.MI_MOE_EALIGN):
             check(rc)
+        _warn_once("weight_kn", f"scattered_gemm(weight_kn=True): the transposed-weight kernel does not take "
+                   f"K={K}, N={N}, E={E}, {inputs.dtype} ({lib.mi_moe_strerror(rc).decode()}); making a transposed "
+                   "copy of the weights for this call")
         weight = weight.transpose(1, 2).contiguous()
     with _stage("scattered_gemm"):
-        check(lib.mi_moe_scattered_gemm_cfg(_ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N,
-                                            E, k, int(grouped_in), int(grouped_out), _code(inputs.dtype), cfg,
-                                            _stream()))
+        rc = _gemm_or_slow(lambda c: lib.mi_moe_scattered_gemm_cfg(
+            _ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N, E, k, int(grouped_in),
+            int(grouped_out), _code(inputs.dtype), c, _stream()), cfg, K, N, inputs.dtype)
+        check(rc)
     return out
+
+
+def _gemm_or_slow(call, cfg: int, K: int, N: int, dtype: torch.dtype) -> int:
+    """Run ``call(cfg)``.  The library refuses 16-bit problems its matrix-core kernels cannot take instead of
+    silently running them on the one-thread-per-output kernel; the reference's op takes any shape, so for an
+    automatic pick (cfg < 0) that refusal is answered here by asking for that kernel explicitly -- with a warning."""
+    rc = call(cfg)
+    if cfg < 0 and rc in (_lib.MI_MOE_EUNSUPPORTED, _lib.MI_MOE_EALIGN):
+        _warn_once("slow_gemm", f"grouped GEMM with K={K}, N={N}, {dtype}: "
+                   f"{_lib.load().mi_moe_strerror(rc).decode()}; running the slow one-thread-per-output kernel "
+                   "(needs K % 8 == 0, N % 4 == 0 and 16-byte aligned tensors for the matrix-core kernels)")
+        rc = call(3)
+    return rc
 
 
 def combine(o: torch.Tensor, gates: torch.Tensor, shared: torch.Tensor | None = None,
@@ -361,9 +388,10 @@ def grouped_wgrad(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor
                   a_idx: torch.Tensor | None = None, b_idx: torch.Tensor | None = None) -> torch.Tensor:
     """dw[e] = sum over the sorted rows r of expert e of outer(a[ai(r)], b[bi(r)]), (E, M, N).
 
-    ``a`` (rows_a, M) and ``b`` (rows_b, N) are 16-bit; ``a_idx`` / ``b_idx`` (L,) int32 map a sorted row to a
-    row of the operand (``None``: the operand is already in sorted order and has L rows).  The per-expert
-    weight gradient of the backward of ``scattered_experts`` (moe.py:91-101)."""
+    ``a`` (rows_a, M) and ``b`` (rows_b, N); ``a_idx`` / ``b_idx`` (L,) int32 map a sorted row to a row of the
+    operand (``None``: the operand is already in sorted order and has L rows).  The per-expert weight gradient of
+    the backward of ``scattered_experts`` (moe.py:91-101).  16-bit operands with M % 8 == N % 8 == 0 run on the
+    matrix cores; fp32 and other shapes on a one-thread-per-element kernel."""
     _dev(a, b, expert_offsets, a_idx, b_idx)
     _no_grad(a, b)
     a = a.contiguous()
@@ -382,8 +410,19 @@ def grouped_wgrad(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor
         L = n
     a_idx = None if a_idx is None else a_idx.contiguous()
     b_idx = None if b_idx is None else b_idx.contiguous()
-    expert_offsets = expert_offsets.contiguous()
+    expert_offsets = _i32(expert_offsets).contiguous()
     lib = _lib.load()
+    if not grouped_wgrad_supported(a, b, E):
+        # fp32 (no matrix-core path for it) and odd shapes: the one-thread-per-element kernel, on the device like
+        # everything else (no per-expert host loop, no synchronisation)
+        if a.dtype != torch.float32:
+            _warn_once("slow_wgrad", f"grouped weight gradient with M={M}, N={N}, E={E}, {a.dtype}: running the slow "
+                       "one-thread-per-element kernel (the matrix-core kernel needs M % 8 == N % 8 == 0, E <= 256)")
+        dw = torch.empty((E, M, N), dtype=a.dtype, device=a.device)
+        with _stage("grouped_wgrad"):
+            check(lib.mi_moe_grouped_wgrad_naive(_ptr(a), _ptr(a_idx), _ptr(b), _ptr(b_idx), _ptr(expert_offsets),
+                                                 _ptr(dw), L, M, N, E, _code(a.dtype), _stream()))
+        return dw
     ws_bytes = int(lib.mi_moe_grouped_wgrad_workspace_bytes(L, E, M, N))
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=a.device)
     dw = torch.empty((E, M, N), dtype=a.dtype, device=a.device)
@@ -483,9 +522,11 @@ def up_swiglu(x: torch.Tensor, w_fc: torch.Tensor, k: int, sorted_scattered_idxs
     if x.shape[0] * k != L:
         raise ValueError("x must have L / k rows")
     act = torch.empty((L, I2 // 2), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
     with _stage("up_swiglu"):
-        check(_lib.load().mi_moe_up_swiglu_cfg(_ptr(x), _ptr(w_fc), _ptr(act), _ptr(ss), _ptr(off), L, H, I2 // 2, E, k,
-                                              _code(x.dtype), cfg, _stream()))
+        check(_gemm_or_slow(lambda c: lib.mi_moe_up_swiglu_cfg(
+            _ptr(x), _ptr(w_fc), _ptr(act), _ptr(ss), _ptr(off), L, H, I2 // 2, E, k, _code(x.dtype), c, _stream()),
+            cfg, H, I2 // 2, x.dtype))
     return act
 
 

@@ -144,6 +144,10 @@ int mi_moe_sort_bin_static(const int32_t* topk_idx, int T, int k, int E, int32_t
  * Replaces: scattered_experts(...) without gates (moe.py:91-101).
  *   in  (in_rows, K), w (E, N, K), out (L, N) of `dtype`; L = T*k rows in sorted order;
  *   expert e owns sorted rows [expert_offsets[e-1], expert_offsets[e]).
+ * F16 / BF16 run on the matrix cores and need K % 8 == 0, N % 4 == 0 (MI_MOE_EUNSUPPORTED otherwise) and `in`, `w`
+ * 16-byte, `out` 8-byte aligned (MI_MOE_EALIGN otherwise); nothing falls back to a slower kernel on its own -- a
+ * caller that wants such a problem computed anyway asks for it with mi_moe_scattered_gemm_cfg(..., cfg = 3).
+ * F32 has only that kernel (one thread per output element) and takes any shape.
  */
 int mi_moe_scattered_gemm(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
                           const int32_t* expert_offsets, int L, int K, int N, int E, int k,
@@ -243,6 +247,13 @@ size_t mi_moe_grouped_wgrad_workspace_bytes(int L, int E, int M, int N);
 int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const void* b, const int32_t* b_idx,
                          const int32_t* expert_offsets, void* dw, void* workspace, size_t workspace_bytes,
                          int L, int a_rows, int b_rows, int M, int N, int E, int dtype, mi_moe_stream_t stream);
+
+/* The same sums for any shape and for F32 as well (the matrix-core kernel above takes 16-bit operands with
+ * M % 8 == N % 8 == 0 only): one thread per element of dw, the expert's rows added in ascending order in fp32, one
+ * rounding.  Slow; no workspace.  M <= 262140, E <= 65535. */
+int mi_moe_grouped_wgrad_naive(const void* a, const int32_t* a_idx, const void* b, const int32_t* b_idx,
+                               const int32_t* expert_offsets, void* dw, int L, int M, int N, int E, int dtype,
+                               mi_moe_stream_t stream);
 
 /*
  * Training-mode auxiliary loss of the router, moe.py:346-369 (one data-parallel rank), and its gradient:
