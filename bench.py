@@ -14,6 +14,9 @@ Zipf(1.1) expert load).  One JSON line is printed:
                     in a second, instrumented run of the same K steps
 * ``cpu_baseline``  the eager per-expert-loop path (the oracle, a port of the reference's eager
                     branch) in fp32 on the host cores, on a bounded token sample of the same workload
+* ``workloads``     (default run only) the other four parity configurations, measured the same way in a few
+                    seconds each: ms per step, the dominant kernel's roofline fraction, both grouped GEMMs
+                    together, and the whole layer's algorithmic bytes over HBM peak (the decode target)
 """
 
 import argparse
@@ -96,6 +99,74 @@ def build_module(w, inputs, device, fp8_tiled=True):
     return m
 
 
+METRIC = "MoE fwd tokens/s & % bf16 MFMA peak, Granite-3B-A800M layer, 1 GPU"  # BASELINE.json, default workload
+
+
+def metric_name(w):
+    if w.name == "granite-3b-a800m":
+        return METRIC
+    what = "% HBM peak" if w.fp8 else "% bf16 MFMA peak"
+    return f"MoE fwd tokens/s & {what}, {w.name} layer, 1 GPU"
+
+
+def layer_algorithmic_bytes(w, touched):
+    """Compulsory HBM traffic of one forward: x once, every touched expert's weights (and fp8 scales) once, the
+    gate weight, y once, and the routing metadata (sorted order: two int32 per slot, gates, offsets)."""
+    elt = 2 if w.dtype != __import__("torch").float32 else 4
+    welt = 1 if w.fp8 else elt
+    L = w.T * w.k
+    weights = touched * (3 * w.I * w.H) * welt + (touched * (2 * w.I + w.H) * 4 if w.fp8 else 0)
+    return w.T * w.H * elt * 2 + weights + w.E * w.H * elt + L * (4 + 4 + elt) + 4 * w.E
+
+
+def measure_compact(name, device, steps=20, warmup=5):
+    """One of the other workloads, timed like the headline: K forwards between two synchronisations, then an
+    instrumented run with HIP events around every stage."""
+    import torch
+
+    from dolomite_engine_amd import Kernel, enable_kernels, ops
+    from oracle import moe_oracle as oracle
+
+    w = oracle.WORKLOADS[name]
+    inputs = oracle.make_inputs(w)
+    m = build_module(w, inputs, device)
+    x = inputs["x"].to(device)
+    L = w.T * w.k
+    with torch.no_grad(), enable_kernels([Kernel.scattermoe]):
+        for _ in range(warmup):
+            m(x)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            m(x)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        timer = StageTimer()
+        ops.set_stage_timer(timer)
+        for _ in range(steps):
+            m(x)
+        stages = timer.summary()
+        ops.set_stage_timer(None)
+        _, _, idx = m._compute_routing_weights(x)
+        touched = int((torch.bincount(idx.flatten().long(), minlength=w.E) > 0).sum())
+    out = {"ms_per_step": ms, "tokens_per_s": w.T / (ms * 1e-3), "dtype": str(w.dtype).replace("torch.", ""),
+           "layer_tflops": 6.0 * L * w.H * w.I / (ms * 1e-3) / 1e12, "stages_ms": stages}
+    layer_bytes = layer_algorithmic_bytes(w, touched)
+    out["layer_hbm_frac"] = layer_bytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS
+    if w.fp8:
+        up_bytes = touched * (2 * w.I * w.H) + touched * 2 * w.I * 4 + w.T * w.H * 2 + L * w.I * 2 + L * 4 + w.E * 4
+        out["kernel"], out["bound"] = "up_swiglu_fp8", "hbm"
+        out["frac"] = up_bytes / (stages["up_swiglu_fp8"] * 1e-3) / 1e9 / PEAK_HBM_GBS
+    elif w.dtype != torch.float32:
+        out["kernel"], out["bound"] = "up_swiglu", "mfma"
+        out["frac"] = 4.0 * L * w.H * w.I / (stages["up_swiglu"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS
+        out["both_gemms_frac"] = (6.0 * L * w.H * w.I / ((stages["up_swiglu"] + stages["scattered_gemm"]) * 1e-3)
+                                  / 1e12 / PEAK_BF16_TFLOPS)
+    del m, x, inputs
+    torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(w, inputs, sample_tokens, iters=3):
     """Eager path of the oracle in fp32 on the host, on the first ``sample_tokens`` tokens."""
     import torch
@@ -151,6 +222,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="granite-3b-a800m")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="default workload only: skip the compact measurements of the other four configurations")
     ap.add_argument("--cpu-sample-tokens", type=int, default=None)
     ap.add_argument("--graph", action="store_true",
                     help="also capture the forward into a HIP graph and report the time of a replay "
@@ -309,7 +382,7 @@ def main():
             roofline["both_gemms_frac"] = flops / ((stages[up_name] + stages["scattered_gemm"]) * 1e-3) / 1e12 / PEAK_BF16_TFLOPS
 
     out = {
-        "metric": "MoE fwd tokens/s & % bf16 MFMA peak, Granite-3B-A800M layer, 1 GPU",
+        "metric": metric_name(w),
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if not w.fp8 else "bf16 activations, fp8-e4m3 weights", "data": "synthetic",
@@ -318,9 +391,14 @@ def main():
                    "experts_touched": touched, "max_over_min_load": float(counts.max()) / max(1.0, float(counts.min())),
                    **({"fp8_weight_layout": "row-major" if args.fp8_row_major else "streamed tiles"} if w.fp8 else {})},
         "layer_tflops": flops / (elapsed / args.steps) / 1e12,
+        "layer_hbm_frac": layer_algorithmic_bytes(w, touched) / (elapsed / args.steps) / 1e9 / PEAK_HBM_GBS,
         "stages_ms": stages,
         "roofline": roofline,
     }
+    if w.name == "granite-3b-a800m" and not args.no_other_workloads:
+        del m, x
+        torch.cuda.empty_cache()
+        out["workloads"] = {n: measure_compact(n, device) for n in oracle.WORKLOADS if n != w.name}
     if graph_ms is not None:
         out["ms_per_step_graph_replay"] = graph_ms
     if train is not None:

@@ -655,46 +655,41 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GemmArgs 
 // XCD's contiguous tile range is dealt to its workgroups in turn, so at any moment the CUs of one XCD
 // work on neighbouring tiles (same expert weights, shared activation rows) out of one L2.
 //
-// PP selects how the eight waves share a SIMD's matrix pipe.  Without it all waves run the same phase
-// and meet at one barrier per K slice: the two waves of a SIMD then stall together (barrier, LDS
-// latency, DMA issue) and the pipe idles.  With it the waves form two groups that alternate between a
-// memory phase and a matrix phase (see pp_slice); measured on the 32768-token Granite-3B shape that
-// takes the K loop from about 65 % to about 93 % matrix-pipe occupancy in cycles.  (With random operands
-// the chip then lowers its clock to stay inside its power limit, so wall time improves less than the
-// cycle count.)
+// The eight waves form two groups that alternate between a memory phase and a matrix phase (see pp_slice).  With
+// all waves in one phase and one barrier per K slice, the two waves of a SIMD stall together (barrier, LDS latency,
+// DMA issue) and the matrix pipe idles: measured on the 32768-token Granite-3B shape, about 65 % matrix-pipe
+// occupancy in cycles inside the K loop against about 80 % for the alternating form, with 32-wide as with 64-wide
+// K slices.  (With random operands the chip then lowers its clock to stay inside its power limit, so wall time
+// improves less than the cycle count.)
 // ------------------------------------------------------------------------------------------------
 
 #define PERSIST_MAX_E 256
 
-template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool PP, bool WT = false>
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool WT = false>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(GemmArgs a) {
-  static_assert(BK == 32 || BK == 64, "BK");
   // WT: the expert weights are (K, N) row-major ("x @ W" with W as stored, the form both data gradients of the
   // backward take).  A K slice of them is 32 rows of 512 bytes; it is staged as it lies in HBM and the fragments
   // are read with the transposing LDS read (see read_frags).
-  static_assert(!WT || (PP && !GLU && BK == 32 && BNW == 256), "transposed-weight form");
-  constexpr int NSTAGE = BK == 32 ? 4 : 2;   // ring of 128 KiB either way
-  constexpr int STEPS = BK / 16;             // MFMA k-steps per ring stage
-  constexpr int RPI = BK == 32 ? 16 : 8;     // stage rows filled by one DMA instruction (1 KiB)
-  constexpr int LROW_SHIFT = BK == 32 ? 2 : 3;  // lane -> row within the instruction's rows
+  static_assert(!WT || (!GLU && BNW == 256), "transposed-weight form");
+  constexpr int BK = 32;                     // K slice per ring stage = one 16x16x32 matrix instruction deep
+  constexpr int NSTAGE = 4;                  // ring of 128 KiB
+  constexpr int RPI = 16;                    // stage rows filled by one DMA instruction (1 KiB)
+  constexpr int LROW_SHIFT = 2;              // lane -> row within the instruction's rows
   constexpr int NW = WM * WN;
   constexpr int ROWS = BM + BNW;
   constexpr int STAGE_BYTES = ROWS * BK * 2;
   constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
-  // per-wave epilogue scratch: 32 rows x EPI_COLS columns.  64 columns make every store a run of whole
-  // 128-byte lines per row (measured: 64-byte pieces write at 4.4-4.6 TB/s chip-wide, 128-byte ones at
-  // 5.0-5.3).  The ping-pong kernel has a free ring stage to put it in; the others carve it out of what is
-  // left of LDS next to a full ring.
-  constexpr int EPI_COLS = (PP || NW <= 4) ? 64 : 32;
+  // per-wave epilogue scratch: 32 rows x 64 columns, in the ring stage that is free at a tile boundary.  64 columns
+  // make every store a run of whole 128-byte lines per row (measured: 64-byte pieces write at 4.4-4.6 TB/s
+  // chip-wide, 128-byte ones at 5.0-5.3).
+  constexpr int EPI_COLS = 64;
   constexpr int EPI_BYTES = 32 * EPI_COLS * 2;
   constexpr int EPI_CPR = EPI_COLS / 8;      // 16-byte chunks per scratch row
   constexpr int NLD = ROWS / RPI / NW;       // DMA instructions per wave per K slice
   constexpr int NXLD = BM / RPI / NW;        // ... of which activation rows (the first NXLD)
   constexpr int BN = GLU ? BNW / 2 : BNW;
   constexpr int WTM = BM / WM, WTN = BNW / WN;
-  // matrix instruction: 32x32x16 (two k steps per 32-wide slice), or with PP 16x16x32 (one step per slice)
-  constexpr int MT = PP ? 16 : 32;           // edge of one accumulator block
-  constexpr int ACC_GROUPS = PP ? 1 : 4;     // 4-register groups per accumulator block
+  constexpr int MT = 16;                     // edge of one accumulator block (v_mfma_f32_16x16x32)
   constexpr int MB = WTM / MT, NB = WTN / MT;
   constexpr int OB = GLU ? NB / 2 : NB;      // output column blocks per wave
   constexpr int EPI_MB = 32 / MT;            // accumulator row blocks per 32-row epilogue pass
@@ -702,13 +697,12 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   static_assert(BM % (16 * NW) == 0 && BNW % (16 * NW) == 0 && NW % 2 == 0, "tile/wave shape");
   static_assert(OB % EPI_NB == 0 && MB % EPI_MB == 0, "epilogue pass shape");
   static_assert((NSTAGE - 1) * NLD <= 63, "vmcnt range");
-  typedef typename Mfma32<T>::vec frag_t;
+  typedef typename Mfma16<T>::vec frag_t;
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
-  typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  // [ring][epilogue scratch: NW x EPI_BYTES, not with PP][expert table: E x (tiles inclusive, row end)]
-  int* etab = reinterpret_cast<int*>(smem_raw + RING_BYTES + (PP ? 0 : NW * EPI_BYTES));
+  // [ring][expert table: E x (tiles inclusive, row end)]
+  int* etab = reinterpret_cast<int*>(smem_raw + RING_BYTES);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -790,13 +784,10 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   const unsigned char* __restrict__ xbase = static_cast<const unsigned char*>(a.in);
   const unsigned char* __restrict__ wall = static_cast<const unsigned char*>(a.w);
   const size_t expert_bytes = (size_t)WROWS_MUL * a.N * a.K * sizeof(T);
-  // logical 16-byte chunk this lane fetches so that it lands in its swizzled slot (see read_frags):
-  //   BK = 32: row = 16*grp + lane/4, slot = lane%4, swizzle (row >> 2) & 3
-  //   BK = 64: row =  8*grp + lane/8, slot = lane%8, swizzle (row & 7) ^ ((row >> 3) & 1); grp parity == wave parity
-  //   PP (16-row fragments over BK = 32): swizzle (row >> 1) & 3 -- the one that reads 16 rows x 4 chunks
-  //   without bank conflicts (measured; (row >> 2) & 3 costs about 20 % of the LDS read rate there)
-  const int lchunk = BK == 32 ? ((lane & 3) ^ (PP ? (lane >> 3) & 3 : (lane >> 4) & 3))
-                              : ((lane & 7) ^ (lane >> 3) ^ (wave & 1));
+  // logical 16-byte chunk this lane fetches so that it lands in its swizzled slot (see read_frags): row =
+  // 16*grp + lane/4, slot = lane%4, swizzle (row >> 1) & 3 -- the one that reads the 16 rows x 4 chunks of a
+  // fragment without bank conflicts (measured; (row >> 2) & 3 costs about 20 % of the LDS read rate there)
+  const int lchunk = (lane & 3) ^ ((lane >> 3) & 3);
   struct TileSrc {
     uint32_t off[NLD];
     const unsigned char* wbase;
@@ -858,10 +849,9 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   };
 
   // ---- fragment reads ----------------------------------------------------------------------------------
-  // lane -> (row of its MT-row block, k chunk): 32x32x16 takes k = 8 * (lane / 32) + [0, 8) of a 16-wide step,
-  // 16x16x32 takes k = 8 * (lane / 16) + [0, 8) of the whole 32-wide slice
+  // lane -> (row of its 16-row block, k chunk): the instruction takes k = 8 * (lane / 16) + [0, 8) of the slice
   const int frow = lane % MT, fhalf = lane / MT;
-  const int fswz = BK == 32 ? (PP ? (frow >> 1) & 3 : (frow >> 2) & 3) : ((frow & 7) ^ ((frow >> 3) & 1));
+  const int fswz = (frow >> 1) & 3;
   int frag_x_off[MB], frag_w_off[NB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) frag_x_off[mb] = (wm * WTM + mb * MT + frow) * (BK * 2);
@@ -877,12 +867,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     }
     frag_w_off[nb] = (BM + r) * (BK * 2);
   }
-  int chunk_byte[STEPS];
-#pragma unroll
-  for (int kk = 0; kk < STEPS; ++kk) chunk_byte[kk] = (((PP ? 0 : 2 * kk) + fhalf) ^ fswz) * 16;
-
-  constexpr int NBUF = PP ? 1 : 2;
-  frag_t xf[NBUF][MB], wf[NBUF][NB];
+  const int chunk_byte = (fhalf ^ fswz) * 16;
+  frag_t xf[MB], wf[NB];
   // WT: ds_read_b64_tr_b16 transposes 4 rows x 16 columns across 16 lanes: lane i of the group supplies the
   // address of (row i / 4, columns 4 (i % 4) ..) and receives column i of the four rows.  Lane group q reads rows
   // 8q .. 8q + 3 and, 2 KiB further, 8q + 4 .. 8q + 7: together the 8 contraction values the matrix instruction
@@ -891,8 +877,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   const int tr_i = lane & 15, tr_q = lane >> 4;
   const uint32_t tr_base = (8 * tr_q + (tr_i >> 2)) * (BNW * 2) + ((((tr_i >> 2) | (tr_q << 2))) << 5) + (tr_i & 3) * 8;
   const uint32_t lds_base = (uint32_t)(size_t)(lds_ptr_t)smem_raw;
-  auto read_frags = [&](int stage, int kk, int buf) {
-    const unsigned char* s = smem_raw + stage * STAGE_BYTES + chunk_byte[kk];
+  auto read_frags = [&](int stage) {
+    const unsigned char* s = smem_raw + stage * STAGE_BYTES + chunk_byte;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
       if constexpr (WT) {
@@ -900,59 +886,36 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
         const uint32_t addr = lds_base + stage * STAGE_BYTES + BM * BK * 2 + (tr_base ^ ((uint32_t)(wn * NB + nb) << 5));
         const tr_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(size_t)addr);
         const tr_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(size_t)(addr + 4 * BNW * 2));
-        wf[buf][nb] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        wf[nb] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
       } else {
-        wf[buf][nb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_w_off[nb]));
+        wf[nb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_w_off[nb]));
       }
     }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
-      xf[buf][mb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_x_off[mb]));
+      xf[mb] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4*>(s + frag_x_off[mb]));
   };
 
-  // accumulator block (nb, mb): register 4 * g + i of a lane is output column MT * nb + 8 * g + 4 * fhalf + i
-  // (weight row) of token row MT * mb + frow
-  typedef typename std::conditional<PP, f32x4, f32x16>::type acc_t;
-  acc_t acc[NB][MB];
+  // accumulator block (nb, mb): register i of a lane is output column 16 * nb + 4 * fhalf + i (weight row) of
+  // token row 16 * mb + frow
+  f32x4 acc[NB][MB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int i = 0; i < 4 * ACC_GROUPS; ++i) acc[nb][mb][i] = 0.f;
+      for (int i = 0; i < 4; ++i) acc[nb][mb][i] = 0.f;
 
-  auto mfma_step = [&](int buf) {
+  // eight instructions in a row share the activation operand
+  auto mfma_step = [&]() {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        if constexpr (PP) acc[nb][mb] = Mfma16<T>::run(wf[buf][nb], xf[buf][mb], acc[nb][mb]);
-        else acc[nb][mb] = Mfma32<T>::run(wf[buf][nb], xf[buf][mb], acc[nb][mb]);
-      }
+      for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mfma16<T>::run(wf[nb], xf[mb], acc[nb][mb]);
   };
 
   int g = 0;  // running K-slice count; slice g lives in ring stage g % NSTAGE
-  // one K slice: consume stage g % NSTAGE, then refill it with slice `kload` of tile cur / next
-  auto slice = [&](const TileSrc& tcur, const TileSrc& tnext, bool from_next, int kload) {
-    const int cur = g & (NSTAGE - 1), nxt = (g + 1) & (NSTAGE - 1);
-#pragma unroll
-    for (int st = 0; st < STEPS - 1; ++st) {
-      read_frags(cur, st + 1, (st + 1) & 1);
-      mfma_step(st & 1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm((NSTAGE - 2) * NLD, 0));
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(nxt, 0, 0);
-    dma_slice(tcur, tnext, from_next, kload, cur);
-    mfma_step((STEPS - 1) & 1);
-    __builtin_amdgcn_sched_barrier(0);
-    ++g;
-  };
-  // Ping-pong form of one K slice (PP; BK = 32, four stages).  The waves with wn == 0 and those with
+  // One K slice.  The waves with wn == 0 and those with
   // wn == 1 -- one of each per SIMD -- run this same code one phase apart (see the tile loop): while one group
   // issues its NB * MB matrix instructions back to back out of registers, the other reads its fragments of the
   // slice from LDS and issues its share of the DMA for slice g + 3 into the stage both groups have finished
@@ -961,7 +924,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   // barrier itself.
   auto pp_slice = [&](const TileSrc& tcur, const TileSrc& tnext, bool from_next, int kload) {
     const int cur = g & (NSTAGE - 1), fill = (g + NSTAGE - 1) & (NSTAGE - 1);
-    read_frags(cur, 0, 0);
+    read_frags(cur);
     dma_slice(tcur, tnext, from_next, kload, fill);
     asm volatile("" ::: "memory");
     // own DMA of slice g + 1 has landed (slices g + 2 and g + 3 stay in flight); fragments are in registers
@@ -971,7 +934,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     __builtin_amdgcn_sched_barrier(0);
     // (Signalling the second barrier a few matrix instructions early, so that they cover its release
     // latency, measured slower: the group's next memory phase then starts late and becomes the long one.)
-    mfma_step(0);
+    mfma_step();
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -980,7 +943,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
 
   // ---- epilogue of one tile: acc -> (SwiGLU) -> LDS scratch -> 16-byte row-contiguous stores -----------
   T* __restrict__ out = static_cast<T*>(a.out);
-  static_assert(!PP || NW * EPI_BYTES <= STAGE_BYTES, "epilogue scratch must fit the free ring stage");
+  static_assert(NW * EPI_BYTES <= STAGE_BYTES, "epilogue scratch must fit the free ring stage");
   constexpr int RPP = 64 / EPI_CPR;  // rows per read-back pass
   constexpr int MP = MB / EPI_MB;    // 32-row passes over the wave's token rows
   // Destination rows of everything this lane will store in a tile's epilogue.  With scattered output they are
@@ -999,20 +962,19 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
       }
   };
   auto epilogue = [&](const TileCoord& tc, const OutRows& orows) {
-    // PP: the ring stage consumed last is free until the next tile's first memory phase refills it (the
-    // tile loop puts a barrier between this epilogue and that refill)
-    unsigned char* scratch = PP ? smem_raw + ((g + NSTAGE - 1) & (NSTAGE - 1)) * STAGE_BYTES + wave * EPI_BYTES
-                                : smem_raw + RING_BYTES + wave * EPI_BYTES;
+    // the ring stage consumed last is free until the next tile's first memory phase refills it (the tile loop
+    // puts a barrier between this epilogue and that refill)
+    unsigned char* scratch = smem_raw + ((g + NSTAGE - 1) & (NSTAGE - 1)) * STAGE_BYTES + wave * EPI_BYTES;
     // scratch row r keeps its EPI_CPR 16-byte chunks at slots chunk ^ swz(r): the 8-byte writes of a
     // wave and the 16-byte read-back both spread over all banks
-    auto swz = [](int r) { return EPI_CPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3); };
+    auto swz = [](int r) { return (r >> 1) & 7; };
     const auto& orow_of = orows.r;
 #pragma unroll
     for (int mp = 0; mp < MP; ++mp) {
 #pragma unroll
       for (int og = 0; og < OB / EPI_NB; ++og) {
         // write the 32 x EPI_COLS block: a lane holds, per accumulator block, token row frow and the four
-        // output columns 8 * g + 4 * fhalf + [0, 4) of each group g
+        // output columns 4 * fhalf + [0, 4)
 #pragma unroll
         for (int mbb = 0; mbb < EPI_MB; ++mbb) {
           const int mb = mp * EPI_MB + mbb;
@@ -1020,24 +982,21 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
 #pragma unroll
           for (int ob = 0; ob < EPI_NB; ++ob) {
             const int nb = og * EPI_NB + ob;
+            float v[4];
 #pragma unroll
-            for (int gq = 0; gq < ACC_GROUPS; ++gq) {
-              float v[4];
-#pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                if (GLU) {
-                  const float up = acc[nb][mb][gq * 4 + i];
-                  const float gt = acc[nb + NB / 2][mb][gq * 4 + i];
-                  v[i] = up * gt * __builtin_amdgcn_rcpf(1.0f + __expf(-gt));
-                } else {
-                  v[i] = acc[nb][mb][gq * 4 + i];
-                }
+            for (int i = 0; i < 4; ++i) {
+              if (GLU) {
+                const float up = acc[nb][mb][i];
+                const float gt = acc[nb + NB / 2][mb][i];
+                v[i] = up * gt * __builtin_amdgcn_rcpf(1.0f + __expf(-gt));
+              } else {
+                v[i] = acc[nb][mb][i];
               }
-              const int colp = ob * MT + gq * 8 + fhalf * 4;  // column inside the pass
-              const u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
-              *reinterpret_cast<u32x2*>(scratch + srow * (EPI_COLS * 2) + (((colp >> 3) ^ swz(srow)) * 16) +
-                                        ((colp >> 2) & 1) * 8) = p;
             }
+            const int colp = ob * MT + fhalf * 4;  // column inside the pass
+            const u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+            *reinterpret_cast<u32x2*>(scratch + srow * (EPI_COLS * 2) + (((colp >> 3) ^ swz(srow)) * 16) +
+                                      ((colp >> 2) & 1) * 8) = p;
           }
         }
         // read back: lane -> row it*RPP + lane/EPI_CPR, 16-byte chunk lane%EPI_CPR
@@ -1057,7 +1016,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int i = 0; i < 4 * ACC_GROUPS; ++i) acc[nb][mb][i] = 0.f;
+        for (int i = 0; i < 4; ++i) acc[nb][mb][i] = 0.f;
   };
 
   // ---- tile loop -------------------------------------------------------------------------------------------
@@ -1079,31 +1038,23 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   OutRows out_cur, out_next;
   load_out_rows(c0, out_cur);
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
-  constexpr int AHEAD = PP ? NSTAGE - 1 : NSTAGE;  // slices in flight ahead of the one being consumed
-  static_assert(!PP || (BK == 32 && WN == 2), "ping-pong shape");
+  constexpr int AHEAD = NSTAGE - 1;  // slices in flight ahead of the one being consumed
+  static_assert(WN == 2, "two wave groups");
 #pragma unroll
   for (int st = 0; st < AHEAD; ++st) dma_slice(src_cur, src_cur, false, st, st);
   __builtin_amdgcn_s_waitcnt(waitcnt_imm((AHEAD - 1) * NLD, 0));
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  if (!PP) read_frags(0, 0, 0);
 
   for (int i = 0;; ++i) {
-    // the ring runs on into the next tile: the last AHEAD slices refill with its first AHEAD
-    if (PP) {
-      // group wn == 1 runs one phase behind group wn == 0 inside a tile; both leave the tile together
-      if (wn == 1) __builtin_amdgcn_s_barrier();
-      for (int kt = 0; kt < nk; ++kt) {
-        const bool from_next = kt >= nk - AHEAD;
-        pp_slice(src_cur, src_next, from_next, from_next ? kt + AHEAD - nk : kt + AHEAD);
-      }
-      if (wn == 0) __builtin_amdgcn_s_barrier();
-    } else {
-      for (int kt = 0; kt < nk; ++kt) {
-        const bool from_next = kt >= nk - NSTAGE;
-        slice(src_cur, src_next, from_next, from_next ? kt + NSTAGE - nk : kt + NSTAGE);
-      }
+    // the ring runs on into the next tile: the last AHEAD slices refill with its first AHEAD.
+    // group wn == 1 runs one phase behind group wn == 0 inside a tile; both leave the tile together
+    if (wn == 1) __builtin_amdgcn_s_barrier();
+    for (int kt = 0; kt < nk; ++kt) {
+      const bool from_next = kt >= nk - AHEAD;
+      pp_slice(src_cur, src_next, from_next, from_next ? kt + AHEAD - nk : kt + AHEAD);
     }
+    if (wn == 0) __builtin_amdgcn_s_barrier();
     const int t2 = tile_of(i + 2);
     TileCoord c2 = c1;
     if (t2 >= 0) locate(t2, c2);
@@ -1111,12 +1062,10 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     load_rows(c2, raw2);
     load_out_rows(c1, out_next);
     epilogue(c0, out_cur);
-    if (PP) {
-      // every wave is done with its scratch before any wave's DMA of the next tile lands in that stage
-      __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
-      __builtin_amdgcn_s_barrier();
-      asm volatile("" ::: "memory");
-    }
+    // every wave is done with its scratch before any wave's DMA of the next tile lands in that stage
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
     if (t1 < 0) {
       // The compiler folds this exit into the loop's back edge and then assumes, inside the slice loop, that
       // the row-index loads above may still be in flight (nobody consumes them on this path): it would drain
@@ -1207,12 +1156,12 @@ static int launch_dma(GemmArgs a, hipStream_t s) {
   return mi_launch_status();
 }
 
-template <typename T, int BM, int BNW, int WM, int WN, bool GLU, int BK, bool PP, bool WT = false>
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool WT = false>
 static int launch_persistent(GemmArgs a, hipStream_t s) {
   constexpr int BN = GLU ? BNW / 2 : BNW;
   constexpr int NW = WM * WN;
-  const size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T) + (PP ? 0 : (size_t)NW * (NW > 4 ? 2048 : 4096)) + (size_t)a.E * 8;
-  auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, BK, PP, WT>;
+  const size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T) + (size_t)a.E * 8;
+  auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, WT>;
   static std::atomic<uint64_t> lds_ok{0};  // the expert table makes lds vary with E: opt in to the most it can be
   int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok);
   if (rc != MI_MOE_OK) return rc;
@@ -1242,7 +1191,6 @@ static int launch_naive(GemmArgs a, hipStream_t s) {
 //   0 / 1 / 2  register-staged 256x256 / 128x128 / 32x256 (any K % 8 == 0)
 //   3          one thread per output element (any shape, any dtype)
 //   4          DMA-staged 128x128, one tile per workgroup (K % 32 == 0)
-//   5 / 6      persistent DMA-staged 256x256, 8 waves, 32-wide / 64-wide K slices, all waves in one phase
 //   7          persistent DMA-staged 256x256, 8 waves, 32-wide K slices, two wave groups in ping-pong
 template <typename T, bool GLU>
 static int dispatch_cfg(GemmArgs a, int cfg, hipStream_t s) {
@@ -1251,11 +1199,7 @@ static int dispatch_cfg(GemmArgs a, int cfg, hipStream_t s) {
     case 1: return launch_tiled<T, 128, 128, 2, 2, GLU>(a, s);
     case 2: return launch_tiled<T, 32, 256, 1, 4, GLU>(a, s);
     case 4: return a.K % 32 == 0 ? launch_dma<T, 128, 128, 2, 2, GLU>(a, s) : MI_MOE_EUNSUPPORTED;
-    case 5: return persistent_ok(a) ? launch_persistent<T, 256, 256, 4, 2, GLU, 32, false>(a, s) : MI_MOE_EUNSUPPORTED;
-    case 6:
-      return persistent_ok(a) && a.K % 64 == 0 ? launch_persistent<T, 256, 256, 4, 2, GLU, 64, false>(a, s)
-                                               : MI_MOE_EUNSUPPORTED;
-    case 7: return persistent_ok(a) ? launch_persistent<T, 256, 256, 4, 2, GLU, 32, true>(a, s) : MI_MOE_EUNSUPPORTED;
+    case 7: return persistent_ok(a) ? launch_persistent<T, 256, 256, 4, 2, GLU>(a, s) : MI_MOE_EUNSUPPORTED;
     default: return MI_MOE_EUNSUPPORTED;
   }
 }
@@ -1344,8 +1288,8 @@ extern "C" int mi_moe_scattered_gemm_wt(const void* in, const void* w_kn, void* 
   if (!tiled_shape_ok(a, L, false) || !persistent_ok(a)) return MI_MOE_EUNSUPPORTED;
   if (!tiled_aligned(a)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == MI_MOE_BF16) return launch_persistent<bf16_t, 256, 256, 4, 2, false, 32, true, true>(a, s);
-  return launch_persistent<f16_t, 256, 256, 4, 2, false, 32, true, true>(a, s);
+  if (dtype == MI_MOE_BF16) return launch_persistent<bf16_t, 256, 256, 4, 2, false, true>(a, s);
+  return launch_persistent<f16_t, 256, 256, 4, 2, false, true>(a, s);
 }
 
 extern "C" int mi_moe_scattered_gemm(const void* in, const void* w, void* out, const int32_t* sorted_scattered,

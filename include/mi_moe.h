@@ -166,11 +166,10 @@ int mi_moe_scattered_gemm_wt(const void* in, const void* w_kn, void* out, const 
 
 /* Same call with an explicit kernel configuration (tuning / benchmarking / tests): cfg = -1 picks one
  * from the shape; 0 / 1 / 2 = register-staged 256x256 / 128x128 / 32x256 tiles; 3 = one thread per
- * output element (any shape, the only fp32 path); 4 = DMA-staged 128x128 (K % 32 == 0); 5 / 6 =
- * persistent DMA-staged 256x256 with 32- / 64-wide K slices (K % 32 / 64 == 0, K >= 128, N % 8 == 0,
- * E <= 256); 7 = the same tile with 32-wide K slices and the two wave groups of a SIMD alternating
- * between LDS/DMA work and matrix instructions (same shape limits as 5; what -1 picks for large
- * expert loads).  A configuration that does not take the shape returns MI_MOE_EUNSUPPORTED. */
+ * output element (any shape, the only fp32 path); 4 = DMA-staged 128x128 (K % 32 == 0); 7 = persistent
+ * DMA-staged 256x256 tiles with 32-wide K slices and the two wave groups of a SIMD alternating between
+ * LDS/DMA work and matrix instructions (K % 32 == 0, K >= 128, N % 8 == 0, E <= 256; what -1 picks for
+ * large expert loads).  A configuration that does not take the shape returns MI_MOE_EUNSUPPORTED. */
 int mi_moe_scattered_gemm_cfg(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
                               const int32_t* expert_offsets, int L, int K, int N, int E, int k,
                               int grouped_in, int grouped_out, int dtype, int cfg, mi_moe_stream_t stream);
