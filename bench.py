@@ -30,6 +30,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
@@ -105,7 +106,7 @@ METRIC = "MoE fwd tokens/s & % bf16 MFMA peak, Granite-3B-A800M layer, 1 GPU"  #
 def metric_name(w):
     if w.name == "granite-3b-a800m":
         return METRIC
-    what = "% HBM peak" if w.fp8 else "% bf16 MFMA peak"
+    what = "% HBM peak" if w.fp8 else ("% fp32 MFMA peak" if w.dtype == __import__("torch").float32 else "% bf16 MFMA peak")
     return f"MoE fwd tokens/s & {what}, {w.name} layer, 1 GPU"
 
 
@@ -157,11 +158,12 @@ def measure_compact(name, device, steps=20, warmup=5):
         up_bytes = touched * (2 * w.I * w.H) + touched * 2 * w.I * 4 + w.T * w.H * 2 + L * w.I * 2 + L * 4 + w.E * 4
         out["kernel"], out["bound"] = "up_swiglu_fp8", "hbm"
         out["frac"] = up_bytes / (stages["up_swiglu_fp8"] * 1e-3) / 1e9 / PEAK_HBM_GBS
-    elif w.dtype != torch.float32:
+    else:
+        peak = PEAK_FP32_TFLOPS if w.dtype == torch.float32 else PEAK_BF16_TFLOPS
         out["kernel"], out["bound"] = "up_swiglu", "mfma"
-        out["frac"] = 4.0 * L * w.H * w.I / (stages["up_swiglu"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS
+        out["frac"] = 4.0 * L * w.H * w.I / (stages["up_swiglu"] * 1e-3) / 1e12 / peak
         out["both_gemms_frac"] = (6.0 * L * w.H * w.I / ((stages["up_swiglu"] + stages["scattered_gemm"]) * 1e-3)
-                                  / 1e12 / PEAK_BF16_TFLOPS)
+                                  / 1e12 / peak)
     del m, x, inputs
     torch.cuda.empty_cache()
     return out
@@ -310,7 +312,7 @@ def main():
         stages = timer.summary()
         ops.set_stage_timer(None)
 
-        idx = ops.router_fused(x, m.gate.weight, k, bias=m.router_logit_bias)[2]
+        idx = m._compute_routing_weights(x)[2]
         counts = torch.bincount(idx.flatten().long(), minlength=E).cpu()
 
     train = None
@@ -372,20 +374,22 @@ def main():
     else:
         up_name = "up_swiglu"
         up_flops = 4.0 * L * H * I
+        peak = PEAK_FP32_TFLOPS if w.dtype == torch.float32 else PEAK_BF16_TFLOPS
         ach = up_flops / (stages[up_name] * 1e-3) / 1e12
-        roofline = {"kernel": up_name, "bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS,
-                    "unit": "TFLOP/s", "frac": ach / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+        roofline = {"kernel": up_name, "bound": "mfma", "achieved": ach, "peak": peak,
+                    "unit": "TFLOP/s", "frac": ach / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
                     "algorithmic_flops": up_flops, "avg_launch_ms": stages[up_name]}
         if "scattered_gemm" in stages:
             down = 2.0 * L * H * I / (stages["scattered_gemm"] * 1e-3) / 1e12
             roofline["down_gemm_tflops"] = down
-            roofline["both_gemms_frac"] = flops / ((stages[up_name] + stages["scattered_gemm"]) * 1e-3) / 1e12 / PEAK_BF16_TFLOPS
+            roofline["both_gemms_frac"] = flops / ((stages[up_name] + stages["scattered_gemm"]) * 1e-3) / 1e12 / peak
 
     out = {
         "metric": metric_name(w),
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if not w.fp8 else "bf16 activations, fp8-e4m3 weights", "data": "synthetic",
+        "dtype": ("bf16 activations, fp8-e4m3 weights" if w.fp8 else {torch.float32: "f32", torch.bfloat16: "bf16",
+                  torch.float16: "f16"}[w.dtype]), "data": "synthetic",
         "config": {"workload": w.name, "tokens": T, "hidden": H, "experts": E, "top_k": k, "intermediate": I,
                    "expert_load": "zipf(1.1) first-choice" if w.zipf_s else "near-uniform",
                    "experts_touched": touched, "max_over_min_load": float(counts.max()) / max(1.0, float(counts.min())),

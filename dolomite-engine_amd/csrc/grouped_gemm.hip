@@ -40,6 +40,18 @@ template <> struct Mfma32<f16_t> {
   }
 };
 
+// fp32 operands: a 16-byte chunk holds four k values; the lane halves (lane / 32) hold different chunks, so four
+// 32x32x2 instructions -- element i of both operands -- consume the eight k values of a chunk pair.  Which k a
+// lane contributes in which step does not matter as long as both operands use the same assignment.
+template <> struct Mfma32<float> {
+  typedef f32x4 vec;
+  static __device__ __forceinline__ f32x16 run(vec a, vec b, f32x16 c) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[i], c, 0, 0, 0);
+    return c;
+  }
+};
+
 // 16x16x32: half the flops per instruction and the same rate, but a quarter of the accumulator traffic
 // per flop.  Under the chip's power limit (random operands) it sustains about 30 % more throughput than
 // 32x32x16, so the persistent ping-pong kernel uses it.
@@ -150,9 +162,10 @@ __device__ __forceinline__ bool decode_tile(const int32_t* __restrict__ off, int
 
 template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool KTAIL>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
-  constexpr int BK = 64;
+  constexpr int CE = 16 / sizeof(T);        // elements per 16-byte chunk (8 for the 16-bit types, 4 for fp32)
+  constexpr int BK = 8 * CE;                // K tile: 128 bytes per row
   constexpr int NT = WM * WN * 64;
-  constexpr int CPR = BK / 8;               // 16-byte chunks per tile row
+  constexpr int CPR = BK / CE;              // 16-byte chunks per tile row
   constexpr int RS = NT / CPR;              // tile rows covered by one pass of the workgroup
   constexpr int XCH = BM * CPR / NT;        // chunks per thread, activation tile
   constexpr int WCH = BNW * CPR / NT;       // chunks per thread, weight tile
@@ -194,7 +207,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
     int srow = row_begin + r0 + j * RS;
     if (srow > row_end - 1) srow = row_end - 1;  // tail rows re-read the last valid row; never stored
     int src = a.gather ? a.sorted_scattered[srow] / a.kdiv : srow;
-    xoff[j] = (uint32_t)src * (uint32_t)a.K + c * 8;
+    xoff[j] = (uint32_t)src * (uint32_t)a.K + c * CE;
   }
 #pragma unroll
   for (int j = 0; j < WCH; ++j) {
@@ -207,7 +220,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
       col = nt * BN + r;
     }
     if (col > a.N - 1) col = a.N - 1;  // column tail re-reads the last weight row; never stored
-    woff[j] = (uint32_t)(half * a.N + col) * (uint32_t)a.K + c * 8;
+    woff[j] = (uint32_t)(half * a.N + col) * (uint32_t)a.K + c * CE;
   }
 
   // LDS tile layout: row r holds its eight 16-byte chunks at slots  chunk ^ swz(r),
@@ -215,8 +228,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
   // logical chunk fall into distinct bank groups (row parity selects the upper / lower 32 banks).
   // RS % 16 == 0, so all chunks of a thread share one swizzle.
   const int sw_c = c ^ ((r0 & 7) ^ ((r0 >> 3) & 1));
-  const int st_x = (r0 * CPR + sw_c) * 8;              // element offset inside the X tile
-  const int st_w = BM * BK + (r0 * CPR + sw_c) * 8;    // ... inside the W tile (after the X tile)
+  const int st_x = (r0 * CPR + sw_c) * CE;              // element offset inside the X tile
+  const int st_w = BM * BK + (r0 * CPR + sw_c) * CE;    // ... inside the W tile (after the X tile)
 
   u32x4 xreg[XCH], wreg[WCH];
   const int nk = (a.K + BK - 1) / BK;
@@ -225,8 +238,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
     int k0 = kt * BK;
     if (KTAIL) {
       // the last K tile may be partial: out-of-range chunks re-read chunk 0 of the row and are zeroed
-      const bool kvalid = (k0 + c * 8) < a.K;
-      const int koff = kvalid ? k0 : -(c * 8);
+      const bool kvalid = (k0 + c * CE) < a.K;
+      const int koff = kvalid ? k0 : -(c * CE);
 #pragma unroll
       for (int j = 0; j < XCH; ++j) {
         u32x4 v = *reinterpret_cast<const u32x4*>(xbase + xoff[j] + koff);
@@ -278,7 +291,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
   }
   int chunk_off[4];
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) chunk_off[kk] = ((kk * 2 + fhalf) ^ fswz) * 8;
+  for (int kk = 0; kk < 4; ++kk) chunk_off[kk] = ((kk * 2 + fhalf) ^ fswz) * CE;
 
   frag_t xf[2][MB], wf[2][NB];
   auto read_frags = [&](int stage, int kk, int buf) {
@@ -307,7 +320,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
   };
 
   // ---- software pipeline ------------------------------------------------------------------------
-  // Per K tile (4 k-steps of 16), with LDS stages cur / nxt and fragment buffers 0 / 1:
+  // Per K tile (4 k-steps of two chunks each), with LDS stages cur / nxt and fragment buffers 0 / 1:
   //   step 0: MFMA(buf0) | read frags(step1, cur) -> buf1
   //   step 1: MFMA(buf1) | read frags(step2, cur) -> buf0 | write first half of tile kt+1 -> nxt
   //   step 2: MFMA(buf0) | read frags(step3, cur) -> buf1 | write second half            -> nxt
@@ -397,8 +410,12 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
             v[i] = acc[nb][mb][g * 4 + i];
           }
         }
-        u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
-        *reinterpret_cast<u32x2*>(orow_ptr + col) = p;
+        if constexpr (sizeof(T) == 4) {
+          *reinterpret_cast<f32x4*>(orow_ptr + col) = (f32x4){v[0], v[1], v[2], v[3]};
+        } else {
+          u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+          *reinterpret_cast<u32x2*>(orow_ptr + col) = p;
+        }
       }
     }
   }
@@ -1115,7 +1132,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_naive_kernel(GemmArgs a) {
 template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool KTAIL>
 static int launch_tiled_k(GemmArgs a, hipStream_t s) {
   constexpr int BN = GLU ? BNW / 2 : BNW;
-  constexpr size_t lds = 2ull * (BM + BNW) * 64 * sizeof(T);
+  constexpr size_t lds = 2ull * (BM + BNW) * 128;  // two stages of 128-byte rows
   auto kern = grouped_gemm_kernel<T, BM, BNW, WM, WN, GLU, KTAIL>;
   if (lds > 64 * 1024) {
     static std::atomic<uint64_t> lds_ok{0};
@@ -1133,7 +1150,7 @@ static int launch_tiled_k(GemmArgs a, hipStream_t s) {
 
 template <typename T, int BM, int BNW, int WM, int WN, bool GLU>
 static int launch_tiled(GemmArgs a, hipStream_t s) {
-  if (a.K % 64 == 0) return launch_tiled_k<T, BM, BNW, WM, WN, GLU, false>(a, s);
+  if (a.K % (128 / (int)sizeof(T)) == 0) return launch_tiled_k<T, BM, BNW, WM, WN, GLU, false>(a, s);
   return launch_tiled_k<T, BM, BNW, WM, WN, GLU, true>(a, s);
 }
 
@@ -1204,16 +1221,27 @@ static int dispatch_cfg(GemmArgs a, int cfg, hipStream_t s) {
   }
 }
 
-// Shapes the matrix-core kernels take: 16-byte chunks along K, 8-byte output pieces, 32-bit element offsets inside
-// one operand.
-static bool tiled_shape_ok(const GemmArgs& a, int in_rows_bound, bool glu) {
-  if (a.K % 8 != 0 || a.N % 4 != 0) return false;
+// fp32 runs on the register-staged kernels only (32x32x2 matrix instructions)
+template <bool GLU>
+static int dispatch_cfg_f32(GemmArgs a, int cfg, hipStream_t s) {
+  switch (cfg) {
+    case 0: return launch_tiled<float, 256, 256, 2, 2, GLU>(a, s);
+    case 1: return launch_tiled<float, 128, 128, 2, 2, GLU>(a, s);
+    case 2: return launch_tiled<float, 32, 256, 1, 4, GLU>(a, s);
+    default: return MI_MOE_EUNSUPPORTED;
+  }
+}
+
+// Shapes the matrix-core kernels take: 16-byte chunks along K (8 elements of a 16-bit type, 4 of fp32), four
+// results per output piece, 32-bit element offsets inside one operand.
+static bool tiled_shape_ok(const GemmArgs& a, int in_rows_bound, bool glu, int elt_bytes) {
+  if (a.K % (16 / elt_bytes) != 0 || a.N % 4 != 0) return false;
   if ((double)in_rows_bound * a.K >= 2147483648.0) return false;
   if ((double)(glu ? 2 : 1) * a.N * a.K >= 2147483648.0) return false;
   return true;
 }
-static bool tiled_aligned(const GemmArgs& a) {
-  return mi_aligned(a.in, 16) && mi_aligned(a.w, 16) && mi_aligned(a.out, 8);
+static bool tiled_aligned(const GemmArgs& a, int elt_bytes) {
+  return mi_aligned(a.in, 16) && mi_aligned(a.w, 16) && mi_aligned(a.out, 4 * elt_bytes);
 }
 
 static int pick_cfg(const GemmArgs& a) {
@@ -1225,23 +1253,28 @@ static int pick_cfg(const GemmArgs& a) {
 }
 
 // cfg < 0 picks a matrix-core kernel from the shape.  Nothing drops to the one-thread-per-output kernel on its own:
-// a 16-bit problem the matrix-core kernels cannot take is refused (MI_MOE_EALIGN for a misaligned pointer,
-// MI_MOE_EUNSUPPORTED for the shape) and the caller asks for cfg 3 explicitly if it wants the slow kernel.  fp32 has
-// no other kernel, so it takes cfg < 0 and cfg 3 alike.
+// a problem the matrix-core kernels cannot take is refused (MI_MOE_EALIGN for a misaligned pointer,
+// MI_MOE_EUNSUPPORTED for the shape) and the caller asks for cfg 3 explicitly if it wants the slow kernel.
 static int run_gemm(GemmArgs a, int dtype, bool glu, int cfg, int in_rows_bound, hipStream_t s) {
   if (a.L == 0) return MI_MOE_OK;
-  const bool half = dtype == MI_MOE_BF16 || dtype == MI_MOE_F16;
-  if (cfg == 3 || !half) {
-    if (cfg >= 0 && cfg != 3) return MI_MOE_EUNSUPPORTED;
+  if (dtype != MI_MOE_F32 && dtype != MI_MOE_F16 && dtype != MI_MOE_BF16) return MI_MOE_EDTYPE;
+  if (cfg == 3) {
     switch (dtype) {
       case MI_MOE_F32: return glu ? launch_naive<float, true>(a, s) : launch_naive<float, false>(a, s);
       case MI_MOE_F16: return glu ? launch_naive<f16_t, true>(a, s) : launch_naive<f16_t, false>(a, s);
-      case MI_MOE_BF16: return glu ? launch_naive<bf16_t, true>(a, s) : launch_naive<bf16_t, false>(a, s);
-      default: return MI_MOE_EDTYPE;
+      default: return glu ? launch_naive<bf16_t, true>(a, s) : launch_naive<bf16_t, false>(a, s);
     }
   }
-  if (!tiled_shape_ok(a, in_rows_bound, glu)) return MI_MOE_EUNSUPPORTED;
-  if (!tiled_aligned(a)) return MI_MOE_EALIGN;
+  const int elt = dtype == MI_MOE_F32 ? 4 : 2;
+  if (!tiled_shape_ok(a, in_rows_bound, glu, elt)) return MI_MOE_EUNSUPPORTED;
+  if (!tiled_aligned(a, elt)) return MI_MOE_EALIGN;
+  if (dtype == MI_MOE_F32) {
+    if (cfg < 0) {
+      const long avg = a.E > 0 ? (long)a.L / a.E : a.L;
+      cfg = avg >= 512 ? 0 : (avg >= 48 ? 1 : 2);
+    }
+    return glu ? dispatch_cfg_f32<true>(a, cfg, s) : dispatch_cfg_f32<false>(a, cfg, s);
+  }
   if (cfg < 0) cfg = pick_cfg(a);
   if (dtype == MI_MOE_BF16) return glu ? dispatch_cfg<bf16_t, true>(a, cfg, s) : dispatch_cfg<bf16_t, false>(a, cfg, s);
   return glu ? dispatch_cfg<f16_t, true>(a, cfg, s) : dispatch_cfg<f16_t, false>(a, cfg, s);
@@ -1285,8 +1318,8 @@ extern "C" int mi_moe_scattered_gemm_wt(const void* in, const void* w_kn, void* 
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = K; a.N = N; a.E = E; a.kdiv = k; a.n_tiles = 0;
   a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1;
-  if (!tiled_shape_ok(a, L, false) || !persistent_ok(a)) return MI_MOE_EUNSUPPORTED;
-  if (!tiled_aligned(a)) return MI_MOE_EALIGN;
+  if (!tiled_shape_ok(a, L, false, 2) || !persistent_ok(a)) return MI_MOE_EUNSUPPORTED;
+  if (!tiled_aligned(a, 2)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == MI_MOE_BF16) return launch_persistent<bf16_t, 256, 256, 4, 2, false, true>(a, s);
   return launch_persistent<f16_t, 256, 256, 4, 2, false, true>(a, s);

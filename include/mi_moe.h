@@ -144,10 +144,11 @@ int mi_moe_sort_bin_static(const int32_t* topk_idx, int T, int k, int E, int32_t
  * Replaces: scattered_experts(...) without gates (moe.py:91-101).
  *   in  (in_rows, K), w (E, N, K), out (L, N) of `dtype`; L = T*k rows in sorted order;
  *   expert e owns sorted rows [expert_offsets[e-1], expert_offsets[e]).
- * F16 / BF16 run on the matrix cores and need K % 8 == 0, N % 4 == 0 (MI_MOE_EUNSUPPORTED otherwise) and `in`, `w`
- * 16-byte, `out` 8-byte aligned (MI_MOE_EALIGN otherwise); nothing falls back to a slower kernel on its own -- a
- * caller that wants such a problem computed anyway asks for it with mi_moe_scattered_gemm_cfg(..., cfg = 3).
- * F32 has only that kernel (one thread per output element) and takes any shape.
+ * All three types run on the matrix cores (F32 with 32x32x2 instructions, fp32 accumulation throughout) and need
+ * 16-byte chunks along K -- K % 8 == 0 for F16 / BF16, K % 4 == 0 for F32 --, N % 4 == 0 (MI_MOE_EUNSUPPORTED
+ * otherwise), `in` and `w` 16-byte aligned and `out` aligned to four elements (MI_MOE_EALIGN otherwise); nothing
+ * falls back to a slower kernel on its own -- a caller that wants such a problem computed anyway asks for the
+ * one-thread-per-output kernel with mi_moe_scattered_gemm_cfg(..., cfg = 3).
  */
 int mi_moe_scattered_gemm(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
                           const int32_t* expert_offsets, int L, int K, int N, int E, int k,
@@ -165,11 +166,12 @@ int mi_moe_scattered_gemm_wt(const void* in, const void* w_kn, void* out, const 
                              int grouped_out, int dtype, mi_moe_stream_t stream);
 
 /* Same call with an explicit kernel configuration (tuning / benchmarking / tests): cfg = -1 picks one
- * from the shape; 0 / 1 / 2 = register-staged 256x256 / 128x128 / 32x256 tiles; 3 = one thread per
- * output element (any shape, the only fp32 path); 4 = DMA-staged 128x128 (K % 32 == 0); 7 = persistent
+ * from the shape; 0 / 1 / 2 = register-staged 256x256 / 128x128 / 32x256 tiles (all three element types);
+ * 3 = one thread per output element (any shape); 4 = DMA-staged 128x128 (K % 32 == 0); 7 = persistent
  * DMA-staged 256x256 tiles with 32-wide K slices and the two wave groups of a SIMD alternating between
  * LDS/DMA work and matrix instructions (K % 32 == 0, K >= 128, N % 8 == 0, E <= 256; what -1 picks for
- * large expert loads).  A configuration that does not take the shape returns MI_MOE_EUNSUPPORTED. */
+ * large expert loads); 4 and 7 are F16 / BF16 only.  A configuration that does not take the shape or type
+ * returns MI_MOE_EUNSUPPORTED. */
 int mi_moe_scattered_gemm_cfg(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
                               const int32_t* expert_offsets, int L, int K, int N, int E, int k,
                               int grouped_in, int grouped_out, int dtype, int cfg, mi_moe_stream_t stream);
