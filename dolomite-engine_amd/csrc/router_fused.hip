@@ -11,6 +11,7 @@
 //   * top-k: a token's 64 candidates live in 4 lanes x 16 registers; each of the k rounds takes a
 //     per-lane maximum of 64-bit keys (ordered value << 32 | ~expert) and a 2-step butterfly.
 #include "common.h"
+#include "sort_block.h"
 
 template <typename T> struct RMfma;
 template <> struct RMfma<bf16_t> {
@@ -451,10 +452,12 @@ __global__ __launch_bounds__(1024) void router_fused_small_kernel(const T* __res
 template <typename T>
 __global__ __launch_bounds__(ROUTER_SPLIT_WAVES * 64) void router_splitk_partial_kernel(
     const T* __restrict__ x, const T* __restrict__ gw, int Trows, int H, int E, int steps_per_split,
-    f32x4* __restrict__ partial) {
+    f32x4* __restrict__ partial, unsigned* __restrict__ ticket) {
   typedef typename RMfma<T>::vec frag_t;
   __shared__ f32x4 red[ROUTER_SPLIT_WAVES][4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // the finish kernel's ticket counter (fused sort) starts at zero: this kernel is complete before that one starts
+  if (ticket != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *ticket = 0u;
   const int r = lane & 15, q = lane >> 4;
   const int tg = blockIdx.x, ks = blockIdx.y;
   int t = tg * 16 + r;
@@ -543,6 +546,52 @@ __global__ __launch_bounds__(256) void router_splitk_finish_kernel(const f32x4* 
   router_epilogue<T>(acc, t, t < Trows, q, bias, E, k, logits_out, gates, idx);
 }
 
+// The finish kernel with the expert sort folded in (few tokens, T * k <= SORT_SINGLE_BLOCK_MAX): every workgroup
+// publishes its 16 tokens' experts and takes a ticket; the workgroup that draws the last ticket sorts all T * k ids
+// in the same launch (the single-block counting sort of routing.hip).  One launch boundary less on a path that is a
+// chain of short dependent launches.  `ticket` is a counter in the workspace that the partial kernel has zeroed.
+template <typename T>
+__global__ __launch_bounds__(256) void router_splitk_finish_sort_kernel(
+    const f32x4* __restrict__ partial, int splits, const float* __restrict__ bias, int Trows, int E, int k, int nbits,
+    T* __restrict__ logits_out, T* __restrict__ gates, int32_t* __restrict__ idx, unsigned* __restrict__ ticket,
+    int32_t* __restrict__ sorted_expert, int32_t* __restrict__ sorted_scattered, int32_t* __restrict__ expert_offsets) {
+  __shared__ f32x4 red[4][4][64];
+  __shared__ int is_last;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int tg = blockIdx.x;
+  const int t = tg * 16 + r;
+  f32x4 acc[4];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) acc[eb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int ks = wave; ks < splits; ks += 4) {
+    const f32x4* src = partial + ((size_t)ks * gridDim.x + tg) * 4 * 64;
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) acc[eb] += src[eb * 64 + lane];
+  }
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) red[wave][eb][lane] = acc[eb];
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) {
+      f32x4 sum = red[0][eb][lane];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) sum += red[w][eb][lane];
+      acc[eb] = sum;
+    }
+    router_epilogue<T>(acc, t, t < Trows, q, bias, E, k, logits_out, gates, idx);
+    __threadfence();  // this workgroup's experts are visible device-wide before its ticket is
+    if (lane == 0) is_last = atomicAdd(ticket, 1u) == gridDim.x - 1;
+  }
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();  // ... and the last workgroup reads what the others published
+  sort_single_block(idx, Trows * k, E, nbits, sorted_expert, sorted_scattered, expert_offsets,
+                    reinterpret_cast<int*>(&red[0][0][0]));
+}
+
 // K splits for the few-token path: one 64-wide K step per wave and round, enough workgroups to occupy the chip
 static int router_splits(int T_, int H) {
   const int steps = mi_ceil_div(H, 64);
@@ -565,7 +614,7 @@ static int launch_router_splitk(const void* x, const void* gw, const float* bias
   const int groups = mi_ceil_div(T_, 16);
   hipLaunchKernelGGL((router_splitk_partial_kernel<T>), dim3(groups, splits), dim3(ROUTER_SPLIT_WAVES * 64), 0, s,
                      static_cast<const T*>(x), static_cast<const T*>(gw), T_, H, E, steps_per_split,
-                     static_cast<f32x4*>(ws));
+                     static_cast<f32x4*>(ws), static_cast<unsigned*>(nullptr));
   int rc = mi_launch_status();
   if (rc != MI_MOE_OK) return rc;
   hipLaunchKernelGGL((router_splitk_finish_kernel<T>), dim3(groups), dim3(256), 0, s, static_cast<const f32x4*>(ws),
@@ -614,6 +663,59 @@ static int launch_router(const void* x, const void* gw, const float* bias, int T
                      static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out),
                      static_cast<T*>(gates), idx);
   return mi_launch_status();
+}
+
+// [partial logits][ticket, padded to 256 bytes]
+static size_t router_sort_ws_bytes(int T_, int H, int k) {
+  const size_t base = router_ws_bytes(T_, H);
+  if (base == 0 || (long)T_ * k > SORT_SINGLE_BLOCK_MAX) return 0;
+  return base + 256;
+}
+
+template <typename T>
+static int launch_router_splitk_sort(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
+                                     void* logits_out, void* gates, int32_t* idx, int32_t* sorted_expert,
+                                     int32_t* sorted_scattered, int32_t* expert_offsets, void* ws, hipStream_t s) {
+  const int splits = router_splits(T_, H);
+  const int steps_per_split = mi_ceil_div(mi_ceil_div(H, 64), splits);
+  const int groups = mi_ceil_div(T_, 16);
+  unsigned* ticket = reinterpret_cast<unsigned*>(static_cast<unsigned char*>(ws) + router_ws_bytes(T_, H));
+  hipLaunchKernelGGL((router_splitk_partial_kernel<T>), dim3(groups, splits), dim3(ROUTER_SPLIT_WAVES * 64), 0, s,
+                     static_cast<const T*>(x), static_cast<const T*>(gw), T_, H, E, steps_per_split,
+                     static_cast<f32x4*>(ws), ticket);
+  int rc = mi_launch_status();
+  if (rc != MI_MOE_OK) return rc;
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  hipLaunchKernelGGL((router_splitk_finish_sort_kernel<T>), dim3(groups), dim3(256), 0, s,
+                     static_cast<const f32x4*>(ws), splits, bias, T_, E, k, nbits, static_cast<T*>(logits_out),
+                     static_cast<T*>(gates), idx, ticket, sorted_expert, sorted_scattered, expert_offsets);
+  return mi_launch_status();
+}
+
+extern "C" size_t mi_moe_router_fused_sort_workspace_bytes(int T, int H, int E, int k) {
+  (void)E;
+  return (T < 1 || H < 1 || k < 1) ? 0 : router_sort_ws_bytes(T, H, k);
+}
+
+extern "C" int mi_moe_router_fused_sort(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,
+                                        int dtype, void* logits_out, void* gates_out, int32_t* idx_out,
+                                        int32_t* sorted_expert, int32_t* sorted_scattered, int32_t* expert_offsets,
+                                        void* ws, size_t ws_bytes, mi_moe_stream_t stream) {
+  if (T < 1 || H < 1 || E < 1 || k < 1 || k > E) return MI_MOE_ESHAPE;
+  if (E > 64 || k > ROUTER_KMAX || H % 16 != 0) return MI_MOE_EUNSUPPORTED;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  const size_t need = router_sort_ws_bytes(T, H, k);
+  if (need == 0) return MI_MOE_EUNSUPPORTED;  // too many tokens for the split-K router or the one-block sort
+  if (!x || !gate_w || !gates_out || !idx_out || !sorted_expert || !sorted_scattered || !expert_offsets) return MI_MOE_ENULL;
+  if (!ws || ws_bytes < need) return MI_MOE_EWORKSPACE;
+  if (!mi_aligned(x, 16) || !mi_aligned(gate_w, 16) || !mi_aligned(ws, 16)) return MI_MOE_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MI_MOE_BF16)
+    return launch_router_splitk_sort<bf16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, sorted_expert,
+                                             sorted_scattered, expert_offsets, ws, s);
+  return launch_router_splitk_sort<f16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, sorted_expert,
+                                          sorted_scattered, expert_offsets, ws, s);
 }
 
 extern "C" size_t mi_moe_router_fused_workspace_bytes(int T, int H, int E) {

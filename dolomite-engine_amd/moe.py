@@ -236,6 +236,15 @@ class MoE(nn.Module):
             residual = residual.reshape(-1, self.hidden_size)
 
         routed = None
+        presorted = None
+        if pre_norm is None and self._use_fused_router(hidden_states) and ops.router_fused_sort_supported(
+            hidden_states, self.num_experts, self.top_k
+        ):
+            # small batch (decode): the router's finishing launch sorts the experts as well
+            _, router_weights, selected_experts, *presorted = ops.router_fused_sort(
+                hidden_states, self.gate.weight, self.top_k, bias=self.router_logit_bias
+            )
+            routed = (None, router_weights, selected_experts)
         if pre_norm is not None:
             norm_weight, norm_eps = pre_norm
             if self._use_fused_router(hidden_states) and ops.rmsnorm_router_fused_supported(
@@ -262,9 +271,9 @@ class MoE(nn.Module):
         if fuse_tail:
             shared = None if self.shared_intermediate_size is None else self._compute_shared_experts(hidden_states)
             hidden_states = self._compute_experts(hidden_states, router_weights, selected_experts,
-                                                  tail=(shared, residual, residual_scale))
+                                                  tail=(shared, residual, residual_scale), presorted=presorted)
         else:
-            moe_output = self._compute_experts(hidden_states, router_weights, selected_experts)
+            moe_output = self._compute_experts(hidden_states, router_weights, selected_experts, presorted=presorted)
             if self.shared_intermediate_size is None:
                 hidden_states = moe_output
             else:
@@ -341,11 +350,16 @@ class MoE(nn.Module):
         return router_logits, router_weights, selected_experts
 
     def _compute_experts(self, hidden_states: torch.Tensor, router_weights: torch.Tensor,
-                         selected_experts: torch.Tensor, tail: tuple | None = None) -> torch.Tensor:
-        """``tail`` = (shared-expert output, residual, residual_scale) to fold into the combine (kernel branch)."""
+                         selected_experts: torch.Tensor, tail: tuple | None = None,
+                         presorted: list | None = None) -> torch.Tensor:
+        """``tail`` = (shared-expert output, residual, residual_scale) to fold into the combine (kernel branch);
+        ``presorted`` = (sorted_expert_idxs, sorted_scattered_idxs, expert_offsets) when the router already
+        produced them."""
         if is_kernel_allowed(Kernel.scattermoe):
             shared, residual, residual_scale = tail if tail is not None else (None, None, None)
-            sorted_expert_idxs, sorted_scattered_idxs, expert_offsets = ops.sort_bin(selected_experts, self.num_experts)
+            sorted_expert_idxs, sorted_scattered_idxs, expert_offsets = (
+                presorted if presorted else ops.sort_bin(selected_experts, self.num_experts)
+            )
 
             if self.c_fc.weight_q is None and self._fused_swiglu and self._needs_grad(hidden_states):
                 # training: the same forward kernels inside a differentiable function (autograd.py)

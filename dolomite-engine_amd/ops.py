@@ -163,6 +163,45 @@ def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch
     return logits, gates, idx
 
 
+def router_fused_sort_supported(x: torch.Tensor, num_experts: int, k: int) -> bool:
+    """Small batches only (the split-K router and the one-block sort): T <= 1024 and T * k <= 8192."""
+    if not (router_fused_supported(x, num_experts, k) and x.is_cuda and x.dim() == 2 and x.shape[0] >= 1):
+        return False
+    return _lib.load().mi_moe_router_fused_sort_workspace_bytes(x.shape[0], x.shape[1], num_experts, k) > 0
+
+
+def router_fused_sort(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch.Tensor | None = None,
+                      return_logits: bool = False):
+    """:func:`router_fused` and :func:`sort_bin` in two launches instead of three (the router's finishing launch
+    sorts as well).  Returns (logits or None, gates (T, k), experts (T, k) int32, sorted_expert_idxs (L,),
+    sorted_scattered_idxs (L,), expert_offsets (E,)), identical to the separate calls."""
+    _dev(x, gate_weight, bias)
+    _no_grad(x, gate_weight)
+    x = x.contiguous()
+    gate_weight = gate_weight.contiguous()
+    T, H = x.shape
+    E = gate_weight.shape[0]
+    if gate_weight.dtype != x.dtype or gate_weight.shape[1] != H:
+        raise ValueError("gate weight must be (E, H) in the dtype of x")
+    if bias is not None:
+        bias = bias.to(torch.float32).contiguous()
+    dev = x.device
+    logits = torch.empty((T, E), dtype=x.dtype, device=dev) if return_logits else None
+    gates = torch.empty((T, k), dtype=x.dtype, device=dev)
+    idx = torch.empty((T, k), dtype=torch.int32, device=dev)
+    se = torch.empty(T * k, dtype=torch.int32, device=dev)
+    ss = torch.empty(T * k, dtype=torch.int32, device=dev)
+    off = torch.empty(E, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    ws_bytes = lib.mi_moe_router_fused_sort_workspace_bytes(T, H, E, k)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    with _stage("router_fused_sort"):
+        check(lib.mi_moe_router_fused_sort(_ptr(x), _ptr(gate_weight), _ptr(bias), T, H, E, k, _code(x.dtype),
+                                          _ptr(logits), _ptr(gates), _ptr(idx), _ptr(se), _ptr(ss), _ptr(off),
+                                          _ptr(ws), ws_bytes, _stream()))
+    return logits, gates, idx, se, ss, off
+
+
 def rmsnorm_router_fused_supported(x: torch.Tensor, num_experts: int, k: int) -> bool:
     return (x.dtype in (torch.bfloat16, torch.float16) and x.is_cuda
             and bool(_lib.load().mi_moe_rmsnorm_router_fused_supported(x.shape[-1], num_experts, k, _code(x.dtype))))

@@ -85,6 +85,20 @@ int mi_moe_router_fused(const void* x, const void* gate_w, const float* bias, in
                         size_t ws_bytes, mi_moe_stream_t stream);
 
 /*
+ * Fused router followed by the expert sort / bin of mi_moe_sort_bin, for small batches (decode): the launch that
+ * finishes the router also sorts (its last workgroup to finish does), one launch boundary less in a chain of short
+ * dependent launches.  Replaces: MoE._compute_routing_weights + the sort / bincount / cumsum of the scatter branch
+ * (moe.py:246-257, 263-271).  Same outputs as the two separate calls, bit for bit.
+ * Taken when mi_moe_router_fused_sort_workspace_bytes(T, H, E, k) is non-zero: T <= 1024 and T * k <= 8192 (and the
+ * limits of mi_moe_router_fused); MI_MOE_EUNSUPPORTED otherwise.  ws: that many bytes, 16-byte aligned.
+ */
+size_t mi_moe_router_fused_sort_workspace_bytes(int T, int H, int E, int k);
+int mi_moe_router_fused_sort(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,
+                             int dtype, void* logits_out, void* gates_out, int32_t* idx_out, int32_t* sorted_expert,
+                             int32_t* sorted_scattered, int32_t* expert_offsets, void* ws, size_t ws_bytes,
+                             mi_moe_stream_t stream);
+
+/*
  * RMSNorm + fused router: x_norm = round(h * rsqrt(mean(h^2) + eps) * ln_weight) (computed in fp32, one rounding,
  * as torch.nn.RMSNorm does), written to x_norm_out, then the fused router above on x_norm -- in one kernel.
  * Replaces: ln_2 of the transformer block followed by MoE._compute_routing_weights

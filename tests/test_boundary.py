@@ -72,6 +72,13 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_router_fused(None, None, None, 4, 64, 8, 2, _lib.F32, None, None, None, None, 0, None) == E_DTYPE
     assert lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) > 0
     assert lib.mi_moe_router_fused_workspace_bytes(32768, 1536, 40) == 0
+    assert lib.mi_moe_router_fused_sort_workspace_bytes(64, 4096, 64, 6) == lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) + 256
+    assert lib.mi_moe_router_fused_sort_workspace_bytes(2048, 1024, 32, 8) == 0   # too many tokens
+    assert lib.mi_moe_router_fused_sort_workspace_bytes(1024, 1024, 64, 9) == 0   # T * k beyond the one-block sort
+    assert lib.mi_moe_router_fused_sort(None, None, None, 2048, 1024, 32, 8, _lib.BF16, None, None, None, None, None,
+                                        None, None, 0, None) == E_UNSUP
+    assert lib.mi_moe_router_fused_sort(None, None, None, 64, 4096, 64, 6, _lib.BF16, None, None, None, None, None,
+                                        None, None, 0, None) == E_NULL
     assert lib.mi_moe_count(None, -1, 8, None, None) == E_SHAPE
     assert lib.mi_moe_sort_bin(None, 4, 2, 0, None, None, None, None, 0, None) == E_SHAPE
     assert lib.mi_moe_sort_bin(None, 4, 2, 8, None, None, None, None, 0, None) == E_NULL

@@ -183,3 +183,37 @@ def test_rmsnorm_router_fused_unsupported_shapes(device):
     assert not ops.rmsnorm_router_fused_supported(x, 64, 6)       # 64 x 4096 gate weights do not fit in LDS
     assert ops.rmsnorm_router_fused_supported(x, 8, 2)
     assert not ops.rmsnorm_router_fused_supported(x.float(), 8, 2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E,k,bias", [(1, 64, 8, 2, False), (15, 32, 8, 8, False), (64, 4096, 64, 6, False),
+                                          (200, 256, 40, 8, True), (1000, 1024, 32, 8, False), (1024, 512, 64, 8, True),
+                                          (130, 48, 5, 1, False)])
+def test_router_fused_sort_equals_separate_calls(device, dtype, T, H, E, k, bias):
+    """Small batches: the router launch that also sorts must give exactly what the fused router followed by
+    mi_moe_sort_bin gives -- logits, gates, experts, sorted order, offsets -- and the sort must be the oracle's.
+    Called twice, so that a ticket counter left over from the first call would show."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(T * 7 + H + E)
+    x = torch.randn(T, H, generator=g).to(dtype).to(device)
+    w = (torch.randn(E, H, generator=g) * 0.05).to(dtype).to(device)
+    b = torch.randn(E, generator=g).to(device) if bias else None
+    assert ops.router_fused_sort_supported(x, E, k)
+    print(f"router_fused_sort T={T} H={H} E={E} k={k} bias={bias} {dtype}", flush=True)
+    ref_logits, ref_gates, ref_idx = ops.router_fused(x, w, k, bias=b, return_logits=True)
+    ref_se, ref_ss, ref_off = ops.sort_bin(ref_idx, E)
+    for _ in range(2):
+        logits, gates, idx, se, ss, off = ops.router_fused_sort(x, w, k, bias=b, return_logits=True)
+        torch.cuda.synchronize()
+        assert torch.equal(logits, ref_logits) and torch.equal(gates, ref_gates) and torch.equal(idx, ref_idx)
+        assert torch.equal(se, ref_se) and torch.equal(ss, ref_ss) and torch.equal(off, ref_off)
+    ose, oss, ooff = oracle.sort_bin(ref_idx.cpu().long(), E)
+    assert torch.equal(se.cpu().long(), ose) and torch.equal(ss.cpu().long(), oss) and torch.equal(off.cpu().long(), ooff)
+
+
+def test_router_fused_sort_limits(device):
+    ops = _ops()
+    x = torch.zeros(2048, 64, dtype=torch.bfloat16, device=device)
+    assert not ops.router_fused_sort_supported(x, 8, 2)          # more than 1024 tokens
+    assert not ops.router_fused_sort_supported(x[:1024], 64, 9)  # k beyond the fused router
+    assert ops.router_fused_sort_supported(x[:1024], 64, 8)      # 8192 slots: the one-block sort's limit
