@@ -33,14 +33,20 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
-# of this script (scaled by what the counters read for the 256 MiB copy of --pmc-calibration: x2.000
-# for FETCH_SIZE, x1.000 for WRITE_SIZE); the summaries are under profiles/.  A counter cannot be read
-# from inside this process, so the figures are recorded here and are null for other workloads.
-MEASURED_TRAFFIC_BYTES = {
-    "granite-3b-a800m": 1555.8e6 + 268.4e6,   # up-projection GEMM: fetch + write
-    "decode-fp8": 755.8e6 + 1.1e6,            # fp8 up-projection: fetch + write
-}
+def measured_traffic(workload):
+    """HBM-side bytes per launch of the dominant kernel, from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+    summary of this workload (profiles/moe_layer_<workload>.txt: its header gives the commands and the calibration
+    against a 256 MiB copy, its traffic table ends in a line `dominant kernel HBM traffic per launch (bytes): N`).
+    A counter cannot be read from inside this process, so the figure is taken from that file; None without it."""
+    path = os.path.join(ROOT, "profiles", f"moe_layer_{workload}.txt")
+    key = "dominant kernel HBM traffic per launch (bytes):"
+    try:
+        for line in open(path):
+            if line.startswith(key):
+                return float(line[len(key):].split()[0]), os.path.relpath(path, ROOT)
+    except (OSError, ValueError, IndexError):
+        pass
+    return None, None
 
 
 class StageTimer:
@@ -363,12 +369,13 @@ def main():
     flops = 6.0 * L * H * I
     touched = int((counts > 0).sum())
 
+    traffic, traffic_src = measured_traffic(w.name)
     if w.fp8:
         up_name = "up_swiglu_fp8"
         up_bytes = touched * (2 * I * H) + touched * 2 * I * 4 + T * H * 2 + L * I * 2 + L * 4 + E * 4
         ach = up_bytes / (stages[up_name] * 1e-3) / 1e9
         roofline = {"kernel": up_name, "bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": ach / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+                    "frac": ach / PEAK_HBM_GBS, "traffic": traffic, "traffic_source": traffic_src,
                     "algorithmic_bytes": up_bytes,
                     "avg_launch_ms": stages[up_name]}
     else:
@@ -377,7 +384,7 @@ def main():
         peak = PEAK_FP32_TFLOPS if w.dtype == torch.float32 else PEAK_BF16_TFLOPS
         ach = up_flops / (stages[up_name] * 1e-3) / 1e12
         roofline = {"kernel": up_name, "bound": "mfma", "achieved": ach, "peak": peak,
-                    "unit": "TFLOP/s", "frac": ach / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+                    "unit": "TFLOP/s", "frac": ach / peak, "traffic": traffic, "traffic_source": traffic_src,
                     "algorithmic_flops": up_flops, "avg_launch_ms": stages[up_name]}
         if "scattered_gemm" in stages:
             down = 2.0 * L * H * I / (stages["scattered_gemm"] * 1e-3) / 1e12

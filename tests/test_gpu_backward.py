@@ -116,6 +116,12 @@ WGRAD_CASES = [
 ]
 
 
+def _seeded_counts(L, weights, g):
+    """Sizes of E groups that add up to L: L draws from the given weights, from the seeded generator only."""
+    draws = torch.multinomial(weights.double(), L, replacement=True, generator=g)
+    return torch.bincount(draws, minlength=weights.numel())
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("L,E,M,N,rows_other", WGRAD_CASES)
 @pytest.mark.parametrize("gather", ["a", "b", "none", "both"])
@@ -126,7 +132,7 @@ def test_grouped_wgrad(device, dtype, L, E, M, N, rows_other, gather):
     w[torch.rand(E, generator=g) < 0.25] = 0
     if w.sum() == 0:
         w[0] = 1
-    counts = torch.distributions.Multinomial(L, w / w.sum()).sample().long() if L > 1 else torch.tensor([L] + [0] * (E - 1))
+    counts = _seeded_counts(L, w, g)
     offsets = counts.cumsum(0).to(torch.int32)
     assert int(offsets[-1]) == L
     ga, gb = gather in ("a", "both"), gather in ("b", "both")
@@ -261,7 +267,7 @@ def test_grouped_wgrad_full_size(device):
     T, k, E, H, I = 32768, 8, 40, 1536, 512
     L = T * k
     w = 1.0 / torch.arange(1, E + 1, dtype=torch.float64) ** 1.1
-    counts = torch.distributions.Multinomial(L, (w / w.sum()).float()).sample().long()
+    counts = _seeded_counts(L, w, g)
     counts = counts[torch.randperm(E, generator=g)]
     offsets = counts.cumsum(0).to(torch.int32).to(device)
     tok = torch.randint(0, T, (L,), generator=g, dtype=torch.int32).to(device)
@@ -299,7 +305,7 @@ def test_grouped_wgrad_random_shapes(device, seed):
     M = 8 * rnd.choice([1, 5, 32, 33, 40, 260, 300])
     N = 8 * rnd.choice([1, 3, 31, 32, 65])
     g = torch.Generator().manual_seed(seed)
-    counts = torch.distributions.Multinomial(L, torch.rand(E, generator=g).pow(4) + 1e-6).sample().long()
+    counts = _seeded_counts(L, torch.rand(E, generator=g).pow(4) + 1e-6, g)
     offsets = counts.cumsum(0).to(torch.int32)
     rows_other = rnd.choice([1, 17, L])
     a = torch.randn(L, M, generator=g).to(torch.bfloat16)
