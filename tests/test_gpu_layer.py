@@ -127,6 +127,60 @@ def test_layer_reference_test_shape_generic_activation(device):
         torch.testing.assert_close(fast.float(), eager.float(), **tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_layer_edge_batches(device, dtype):
+    """Batches the tile and chunk sizes do not divide: no token at all, one token, the reference test's 15 tokens
+    (test_common.py:96-170), 17, a (batch, sequence, hidden) input and a non-contiguous view of a wider tensor; every
+    one against the oracle on the same logits, and the empty batch returns an empty tensor of the input's shape."""
+    import dataclasses
+
+    from dolomite_engine_amd import Kernel, enable_kernels, ops
+
+    w = dataclasses.replace(oracle.WORKLOADS["tiny-fp32"], dtype=dtype, H=64, I=96, E=8, k=2, name="edge")
+    inputs = oracle.make_inputs(w, T=40)
+    m = _build(w, inputs, device)
+    tol = dict(rtol=1e-3, atol=2e-4) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+    def run(x_dev):
+        with torch.no_grad(), enable_kernels([Kernel.scattermoe]):
+            y = m(x_dev)
+            # the logits of the call the forward itself makes for this batch
+            flat = x_dev.reshape(-1, w.H)
+            if flat.shape[0] and m._use_fused_router(flat) and ops.router_fused_sort_supported(flat, w.E, w.k):
+                logits = ops.router_fused_sort(flat, m.gate.weight, w.k, bias=m.router_logit_bias, return_logits=True)[0]
+            else:
+                logits = m._compute_routing_weights(flat)[0]
+        return y, logits
+
+    for T in (0, 1, 15, 17):
+        print(f"edge batch T={T} {dtype}", flush=True)
+        x = inputs["x"][:T].contiguous()
+        y, logits = run(x.to(device))
+        assert y.shape == x.shape and y.dtype == dtype
+        if T == 0:
+            continue
+        ref = oracle.moe_forward(x, inputs["gate_w"], inputs["w_fc"], inputs["w_proj"], w.k, logits=logits.cpu())
+        assert_close_scaled(y, ref.y, dtype, what=f"edge T={T}", **tol)
+
+    print(f"edge batch 3-D {dtype}", flush=True)
+    x3 = inputs["x"][:21].reshape(3, 7, w.H).contiguous()
+    m.use_padding_free_transformer = False  # (batch, sequence, hidden) in and out, moe.py:213-216, 228-229
+    y3, logits = run(x3.to(device))
+    m.use_padding_free_transformer = True
+    assert y3.shape == x3.shape
+    ref = oracle.moe_forward(x3.reshape(21, w.H), inputs["gate_w"], inputs["w_fc"], inputs["w_proj"], w.k, logits=logits.cpu())
+    assert_close_scaled(y3.reshape(21, w.H), ref.y, dtype, what="edge 3-D", **tol)
+
+    print(f"edge batch non-contiguous {dtype}", flush=True)
+    wide = torch.zeros(40, 2 * w.H, dtype=dtype)
+    wide[:, : w.H] = inputs["x"]
+    view = wide.to(device)[:, : w.H]
+    assert not view.is_contiguous()
+    yv, logits = run(view)
+    ref = oracle.moe_forward(inputs["x"], inputs["gate_w"], inputs["w_fc"], inputs["w_proj"], w.k, logits=logits.cpu())
+    assert_close_scaled(yv, ref.y, dtype, what="edge non-contiguous", **tol)
+
+
 def test_layer_shared_experts(device):
     from dolomite_engine_amd import Kernel, MoE, enable_kernels
 
