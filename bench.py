@@ -106,7 +106,7 @@ def build_module(w, inputs, device, fp8_tiled=True):
     return m
 
 
-METRIC = "MoE fwd tokens/s & % bf16 MFMA peak, Granite-3B-A800M layer, 1 GPU"  # BASELINE.json, default workload
+METRIC = "MoE fwd tokens/s & % bf16 MFMA peak, Granite-3B-A800M layer, 1 GPU"  # the headline metric string, for the default workload
 
 
 def metric_name(w):

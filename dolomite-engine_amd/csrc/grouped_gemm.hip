@@ -84,6 +84,7 @@ struct GemmArgs {
   int gather;   // input row of sorted row i is sorted_scattered[i] / kdiv (else i)
   int scatter;  // output row of sorted row i is sorted_scattered[i] (else i)
   int remap;    // XCD-aware tile order
+  void* ws;     // persistent kernel: workspace for splitting the last round of tiles along K (or null)
 };
 
 
@@ -682,6 +683,104 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GemmArgs 
 
 #define PERSIST_MAX_E 256
 
+// Splitting the last round along K.  A workgroup's tiles all take the same time, so when the tiles of an XCD do not
+// fill its last round, the workgroups without a tile wait for one tile time.  With a workspace, the `rem` tiles of
+// that round are cut into `parts` = min(slots / rem, PERSIST_SPLIT_MAX) ranges of K slices, one per workgroup; a
+// part writes its fp32 accumulators to the workspace instead of running the epilogue, and a second, small launch
+// (grouped_gemm_split_finish_kernel) adds the parts of every split tile in part order and runs the epilogue, so
+// the result does not depend on timing.  A round is only split if that shortens it by at least
+// PERSIST_SPLIT_MIN_SAVED slices: the partial tiles' trip through memory and the second launch cost 40-80 us
+// (measured), about 100 slices' worth.
+#define PERSIST_SPLIT_MAX 4
+#define PERSIST_SPLIT_MIN_SAVED 120
+#define PERSIST_SPLIT_MIN_SLICES 32
+#define PERSIST_WS_TILE_BYTES (256 * 256 * 4)
+
+struct SplitPlan {
+  int per;          // tiles per XCD (the last XCD may have fewer)
+  int full_rounds;  // rounds in which every slot of the XCD has a tile
+  int rem;          // tiles of the last round
+  int parts;        // K ranges each of them is cut into (1: not split)
+};
+
+__device__ __forceinline__ SplitPlan persist_split_plan(int total, int xcd, int nslot, int nk, bool have_ws) {
+  SplitPlan sp;
+  sp.per = (total + 7) >> 3;
+  int n_x = total - xcd * sp.per;
+  n_x = n_x < 0 ? 0 : (n_x < sp.per ? n_x : sp.per);
+  sp.full_rounds = n_x / nslot;
+  sp.rem = n_x - sp.full_rounds * nslot;
+  sp.parts = 1;
+  if (have_ws && sp.rem > 0) {
+    int p = nslot / sp.rem;
+    if (p > PERSIST_SPLIT_MAX) p = PERSIST_SPLIT_MAX;
+    if (p >= 2 && nk / p >= PERSIST_SPLIT_MIN_SLICES && nk - nk / p >= PERSIST_SPLIT_MIN_SAVED) sp.parts = p;
+  }
+  return sp;
+}
+
+// etab[2e] = row tiles of experts 0..e, etab[2e+1] = offsets[e]; filled by the calling wave (all 64 lanes)
+template <int BM>
+__device__ __forceinline__ void persist_expert_table(const int32_t* __restrict__ off, int E, int* etab) {
+  const int lane = threadIdx.x & 63;
+  int carry = 0;
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    const int e = e0 + lane;
+    const int end = e < E ? off[e] : 0;
+    const int prev = (e < E && e > 0) ? off[e - 1] : 0;
+    const int t = e < E ? (end - prev + BM - 1) / BM : 0;
+    int incl = t;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      int v = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += v;
+    }
+    incl += carry;
+    if (e < E) {
+      etab[2 * e] = incl;
+      etab[2 * e + 1] = end;
+    }
+    carry = __shfl(incl, 63, 64);
+  }
+}
+
+// tile id -> coordinates, from the LDS table (wave-uniform result).  An expert's tiles are numbered band
+// by band: a band is up to 8 column tiles wide and runs over all of the expert's row tiles, row tile
+// slowest.  The 32 workgroups of an XCD, which take 32 consecutive tiles at a time, then cover about
+// 4 row tiles x 8 column tiles: 12 operand slabs for 32 tiles, and each weight slab is fetched once per
+// band instead of once per row tile (with many column tiles -- intermediate 14336 -- a plain row-major
+// order re-streams all of an expert's weights from HBM for every row tile).  Up to 8 column tiles the band
+// is the whole row, so that complete output rows are written at about the same time.
+template <int BM>
+__device__ __forceinline__ void persist_locate(const int* etab, int E, int n_tiles, int tile, TileCoord& tc) {
+  const int lane = threadIdx.x & 63;
+  const int tile_band = n_tiles < 8 ? n_tiles : 8;
+  const int q = tile / n_tiles;  // experts own contiguous tile ranges: (row tiles before) * n_tiles
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    const int e = e0 + lane;
+    const int incl = e < E ? etab[2 * e] : 0x7fffffff;
+    const uint64_t hit = __ballot(incl > q);
+    if (hit) {
+      const int ex = e0 + __ffsll((long long)hit) - 1;
+      const int first_tile = ex > 0 ? etab[2 * (ex - 1)] : 0;
+      const int prev = ex > 0 ? etab[2 * (ex - 1) + 1] : 0;
+      const int row_tiles = etab[2 * ex] - first_tile;
+      const int local = tile - first_tile * n_tiles;
+      const int band = local / (row_tiles * tile_band);
+      const int rem = local - band * row_tiles * tile_band;
+      const int left = n_tiles - band * tile_band;
+      const int width = left < tile_band ? left : tile_band;
+      const int mt = rem / width;
+      tc.expert = ex;
+      tc.nt = band * tile_band + rem - mt * width;
+      tc.row_begin = prev + mt * BM;
+      tc.row_end = etab[2 * ex + 1];
+      return;
+    }
+  }
+  tc.expert = 0; tc.nt = 0; tc.row_begin = 0; tc.row_end = 1;  // unreachable for a valid tile id
+}
+
 template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool WT = false>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(GemmArgs a) {
   // WT: the expert weights are (K, N) row-major ("x @ W" with W as stored, the form both data gradients of the
@@ -726,72 +825,32 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   const int wm = wave % WM, wn = wave / WM;
 
   // ---- per-expert table: etab[2e] = row tiles of experts 0..e, etab[2e+1] = offsets[e] ---------------
-  if (wave == 0) {
-    int carry = 0;
-    for (int e0 = 0; e0 < a.E; e0 += 64) {
-      const int e = e0 + lane;
-      const int end = e < a.E ? a.expert_offsets[e] : 0;
-      const int prev = (e < a.E && e > 0) ? a.expert_offsets[e - 1] : 0;
-      const int t = e < a.E ? (end - prev + BM - 1) / BM : 0;
-      int incl = t;
-#pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        int v = __shfl_up(incl, o, 64);
-        if (lane >= o) incl += v;
-      }
-      incl += carry;
-      if (e < a.E) {
-        etab[2 * e] = incl;
-        etab[2 * e + 1] = end;
-      }
-      carry = __shfl(incl, 63, 64);
-    }
-  }
+  if (wave == 0) persist_expert_table<BM>(a.expert_offsets, a.E, etab);
   __syncthreads();
   const int total = etab[2 * (a.E - 1)] * a.n_tiles;
-  const int per = (total + 7) >> 3;
   const int xcd = blockIdx.x & 7, slot0 = blockIdx.x >> 3, nslot = gridDim.x >> 3;
+  const int nk = a.K / BK;  // >= NSTAGE (host-checked)
+  // this XCD's tiles: full_rounds rounds over all slots, then `rem` tiles, each cut into `parts` K ranges
+  const SplitPlan sp = persist_split_plan(total, xcd, nslot, nk, a.ws != nullptr);
+  const int my_part = sp.parts > 1 ? slot0 / sp.rem : 0, my_rem_tile = sp.rem > 0 ? slot0 % sp.rem : 0;
 
   // i-th tile of this workgroup, or -1
   auto tile_of = [&](int i) -> int {
-    const int local = slot0 + i * nslot;
-    const int t = xcd * per + local;
-    return (local < per && t < total) ? t : -1;
+    if (i < sp.full_rounds) return xcd * sp.per + slot0 + i * nslot;
+    if (i > sp.full_rounds || slot0 >= sp.rem * sp.parts) return -1;
+    return xcd * sp.per + sp.full_rounds * nslot + my_rem_tile;
   };
-  // tile id -> coordinates, from the LDS table (wave-uniform result).  An expert's tiles are numbered band
-  // by band: a band is up to 8 column tiles wide and runs over all of the expert's row tiles, row tile
-  // slowest.  The 32 workgroups of an XCD, which take 32 consecutive tiles at a time, then cover about
-  // 4 row tiles x 8 column tiles: 12 operand slabs for 32 tiles, and each weight slab is fetched once per
-  // band instead of once per row tile (with many column tiles -- intermediate 14336 -- a plain row-major
-  // order re-streams all of an expert's weights from HBM for every row tile).  Up to 8 column tiles the band
-  // is the whole row, so that complete output rows are written at about the same time.
-  const int tile_band = a.n_tiles < 8 ? a.n_tiles : 8;
-  auto locate = [&](int tile, TileCoord& tc) {
-    const int q = tile / a.n_tiles;  // experts own contiguous tile ranges: (row tiles before) * n_tiles
-    for (int e0 = 0; e0 < a.E; e0 += 64) {
-      const int e = e0 + lane;
-      const int incl = e < a.E ? etab[2 * e] : 0x7fffffff;
-      const uint64_t hit = __ballot(incl > q);
-      if (hit) {
-        const int ex = e0 + __ffsll((long long)hit) - 1;
-        const int first_tile = ex > 0 ? etab[2 * (ex - 1)] : 0;
-        const int prev = ex > 0 ? etab[2 * (ex - 1) + 1] : 0;
-        const int row_tiles = etab[2 * ex] - first_tile;
-        const int local = tile - first_tile * a.n_tiles;
-        const int band = local / (row_tiles * tile_band);
-        const int rem = local - band * row_tiles * tile_band;
-        const int left = a.n_tiles - band * tile_band;
-        const int width = left < tile_band ? left : tile_band;
-        const int mt = rem / width;
-        tc.expert = ex;
-        tc.nt = band * tile_band + rem - mt * width;
-        tc.row_begin = prev + mt * BM;
-        tc.row_end = etab[2 * ex + 1];
-        return;
-      }
+  // K slices [k0, k0 + len) of the i-th item
+  auto item_k = [&](int i, int& k0, int& len) {
+    if (i == sp.full_rounds && sp.parts > 1) {
+      k0 = my_part * nk / sp.parts;
+      len = (my_part + 1) * nk / sp.parts - k0;
+    } else {
+      k0 = 0;
+      len = nk;
     }
-    tc.expert = 0; tc.nt = 0; tc.row_begin = 0; tc.row_end = 1;  // unreachable for a valid tile id
   };
+  auto locate = [&](int tile, TileCoord& tc) { persist_locate<BM>(etab, a.E, a.n_tiles, tile, tc); };
 
   // ---- DMA sources -----------------------------------------------------------------------------------
   // A tile's sources are NLD 32-bit byte offsets per lane (activation rows relative to the input
@@ -1036,14 +1095,31 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
         for (int i = 0; i < 4; ++i) acc[nb][mb][i] = 0.f;
   };
 
+  // ---- a part of a split tile: accumulators -> workspace (one partial tile per (XCD, slot), fp32) -----------------
+  // Vector j of thread t lies at [j][t]: every store instruction writes 8 KB in a row.  The address is a uniform
+  // base that moves from vector to vector plus one per-thread offset (the accumulators leave no registers for an
+  // address per vector).
+  auto store_part = [&]() {
+    constexpr size_t PART_VECS = (size_t)NB * MB * NW * 64;  // f32x4 per partial tile
+    unsigned t = tid;
+    asm volatile("" : "+v"(t));  // (keeps the offset from being computed ahead of the tile loop and held through it)
+    f32x4* base = static_cast<f32x4*>(a.ws) + ((size_t)xcd * nslot + (size_t)my_rem_tile * sp.parts + my_part) * PART_VECS;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) (base + (nb * MB + mb) * (NW * 64))[t] = acc[nb][mb];
+  };
+
   // ---- tile loop -------------------------------------------------------------------------------------------
-  const int nk = a.K / BK;  // >= NSTAGE (host-checked)
   int t0 = tile_of(0);
   if (t0 < 0) return;
   TileCoord c0, c1;
   locate(t0, c0);
   int t1 = tile_of(1);
   if (t1 >= 0) locate(t1, c1); else c1 = c0;
+  int k0_cur, nk_cur, k0_next, nk_next;
+  item_k(0, k0_cur, nk_cur);
+  if (t1 >= 0) item_k(1, k0_next, nk_next); else { k0_next = k0_cur; nk_next = nk_cur; }
   TileSrc src_cur, src_next;
   {
     int raw0[NXLD], raw1[NXLD];
@@ -1058,7 +1134,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   constexpr int AHEAD = NSTAGE - 1;  // slices in flight ahead of the one being consumed
   static_assert(WN == 2, "two wave groups");
 #pragma unroll
-  for (int st = 0; st < AHEAD; ++st) dma_slice(src_cur, src_cur, false, st, st);
+  for (int st = 0; st < AHEAD; ++st) dma_slice(src_cur, src_cur, false, k0_cur + st, st);
   __builtin_amdgcn_s_waitcnt(waitcnt_imm((AHEAD - 1) * NLD, 0));
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
@@ -1067,11 +1143,16 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     // the ring runs on into the next tile: the last AHEAD slices refill with its first AHEAD.
     // group wn == 1 runs one phase behind group wn == 0 inside a tile; both leave the tile together
     if (wn == 1) __builtin_amdgcn_s_barrier();
-    for (int kt = 0; kt < nk; ++kt) {
-      const bool from_next = kt >= nk - AHEAD;
-      pp_slice(src_cur, src_next, from_next, from_next ? kt + AHEAD - nk : kt + AHEAD);
+    for (int kt = 0; kt < nk_cur; ++kt) {
+      const bool from_next = kt >= nk_cur - AHEAD;
+      pp_slice(src_cur, src_next, from_next, from_next ? k0_next + kt + AHEAD - nk_cur : k0_cur + kt + AHEAD);
     }
     if (wn == 0) __builtin_amdgcn_s_barrier();
+    if (nk_cur != nk) {
+      // a part of a split tile, always a workgroup's last item: the finishing launch adds the parts up
+      store_part();
+      break;
+    }
     const int t2 = tile_of(i + 2);
     TileCoord c2 = c1;
     if (t2 >= 0) locate(t2, c2);
@@ -1095,12 +1176,90 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     t1 = t2;
     src_cur = src_next;
     out_cur = out_next;
+    k0_cur = k0_next;
+    nk_cur = nk_next;
+    if (t2 >= 0) item_k(i + 2, k0_next, nk_next);  // else: the surplus DMA of the last item re-reads its own slices
     make_src(c2, raw2, src_next);
     // Retire every load the compiler knows about (row indices, epilogue traffic) here, once per tile:
     // otherwise it re-checks them with vmcnt(0) inside the slice loop and drains the DMA ring there.
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));  // surplus DMA must not outlive the workgroup's LDS
+}
+
+// The tiles the persistent kernel cut along K (see PERSIST_SPLIT_MAX): one workgroup per (XCD, tile of its last
+// round) recomputes the same plan, adds the tile's partial accumulators in part order and writes the tile the way
+// the persistent kernel's epilogue does (same arithmetic, same rounding; thread t holds what thread t of a part
+// held).  Workgroups whose tile does not exist or was not split return at once.
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU>
+__global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_split_finish_kernel(GemmArgs a, int nslot) {
+  constexpr int NW = WM * WN;
+  constexpr int BN = GLU ? BNW / 2 : BNW;
+  constexpr int WTM = BM / WM, WTN = BNW / WN;
+  constexpr int MT = 16;
+  constexpr int MB = WTM / MT, NB = WTN / MT;
+  constexpr int OB = GLU ? NB / 2 : NB;
+  constexpr size_t PART_VECS = (size_t)NB * MB * NW * 64;
+  __shared__ int etab[2 * PERSIST_MAX_E];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave % WM, wn = wave / WM;
+  if (wave == 0) persist_expert_table<BM>(a.expert_offsets, a.E, etab);
+  __syncthreads();
+  const int total = etab[2 * (a.E - 1)] * a.n_tiles;
+  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  const SplitPlan sp = persist_split_plan(total, xcd, nslot, a.K / 32, true);
+  if (sp.parts == 1 || j >= sp.rem) return;
+  TileCoord tc;
+  persist_locate<BM>(etab, a.E, a.n_tiles, xcd * sp.per + sp.full_rounds * nslot + j, tc);
+
+  // vector j of thread t of a part lies at [j][t]
+  const f32x4* part = static_cast<const f32x4*>(a.ws) + ((size_t)xcd * nslot + (size_t)j * sp.parts) * PART_VECS + tid;
+  f32x4 sum[NB][MB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) sum[nb][mb] = __builtin_nontemporal_load(part + (nb * MB + mb) * (NW * 64));
+  for (int p = 1; p < sp.parts; ++p) {
+    part += PART_VECS;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const f32x4 v = __builtin_nontemporal_load(part + (nb * MB + mb) * (NW * 64));
+#pragma unroll
+        for (int c = 0; c < 4; ++c) sum[nb][mb][c] += v[c];
+      }
+  }
+
+  // accumulator block (nb, mb): register i of a lane is output column 16 * nb + 4 * fhalf + i of the wave's
+  // columns, token row 16 * mb + frow of the wave's rows; with SwiGLU block nb + NB / 2 holds the gate of block nb
+  const int frow = lane % MT, fhalf = lane / MT;
+  T* __restrict__ out = static_cast<T*>(a.out);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int row = tc.row_begin + wm * WTM + mb * MT + frow;
+    if (row >= tc.row_end) continue;
+    const int orow = a.scatter ? a.sorted_scattered[row] : row;
+#pragma unroll
+    for (int nb = 0; nb < OB; ++nb) {
+      const int col = tc.nt * BN + (GLU ? wn * (WTN / 2) : wn * WTN) + nb * MT + fhalf * 4;
+      if (col >= a.N) continue;
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (GLU) {
+          const float up = sum[nb][mb][i];
+          const float gt = sum[nb + NB / 2][mb][i];
+          v[i] = up * gt * __builtin_amdgcn_rcpf(1.0f + __expf(-gt));
+        } else {
+          v[i] = sum[nb][mb][i];
+        }
+      }
+      const u32x2 p2 = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
+      *reinterpret_cast<u32x2*>(out + (size_t)orow * a.N + col) = p2;
+    }
+  }
 }
 
 // ---- any-shape / any-dtype fallback (one thread per output element) ------------------------------
@@ -1177,6 +1336,7 @@ template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool WT = false
 static int launch_persistent(GemmArgs a, hipStream_t s) {
   constexpr int BN = GLU ? BNW / 2 : BNW;
   constexpr int NW = WM * WN;
+  static_assert(BM * BNW * 4 == PERSIST_WS_TILE_BYTES, "size of a partial tile in the workspace");
   const size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T) + (size_t)a.E * 8;
   auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, WT>;
   static std::atomic<uint64_t> lds_ok{0};  // the expert table makes lds vary with E: opt in to the most it can be
@@ -1188,8 +1348,32 @@ static int launch_persistent(GemmArgs a, hipStream_t s) {
   long max_tiles = ((long)a.L / BM + (a.E < a.L ? a.E : a.L)) * a.n_tiles;
   long grid = cus < max_tiles ? cus : max_tiles;
   grid = (grid + 7) / 8 * 8;
+  // no contraction length that a split could shorten by PERSIST_SPLIT_MIN_SAVED slices, or one slot per XCD
+  {
+    const int nk = a.K / 32;
+    if (nk - nk / PERSIST_SPLIT_MAX < PERSIST_SPLIT_MIN_SAVED || grid < 16) a.ws = nullptr;
+  }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, a);
+  if ((rc = mi_launch_status()) != MI_MOE_OK || a.ws == nullptr) return rc;
+  // the tiles that were cut: at most half of an XCD's slots hold tiles of a split round
+  const int nslot = (int)(grid / 8);
+  hipLaunchKernelGGL((grouped_gemm_split_finish_kernel<T, BM, BNW, WM, WN, GLU>), dim3(8u * (unsigned)(nslot / 2)),
+                     dim3(NW * 64), 0, s, a, nslot);
   return mi_launch_status();
+}
+
+// workspace of the persistent kernel: one fp32 partial tile per workgroup of the largest grid
+extern "C" size_t mi_moe_grouped_gemm_workspace_bytes(void) {
+  int cus = 0;
+  if (mi_cu_count(&cus) != MI_MOE_OK) return 0;
+  return (size_t)((cus + 7) / 8 * 8) * PERSIST_WS_TILE_BYTES;
+}
+
+static int check_ws(const void* ws, size_t ws_bytes) {
+  if (ws == nullptr) return MI_MOE_OK;
+  const size_t need = mi_moe_grouped_gemm_workspace_bytes();
+  if (need == 0 || ws_bytes < need) return MI_MOE_EWORKSPACE;
+  return mi_aligned(ws, 16) ? MI_MOE_OK : MI_MOE_EALIGN;
 }
 
 static bool persistent_ok(const GemmArgs& a) {
@@ -1290,39 +1474,57 @@ static int check_common(const void* in, const void* w, void* out, const int32_t*
   return MI_MOE_OK;
 }
 
-extern "C" int mi_moe_scattered_gemm_cfg(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
-                                         const int32_t* expert_offsets, int L, int K, int N, int E, int k,
-                                         int grouped_in, int grouped_out, int dtype, int cfg,
-                                         mi_moe_stream_t stream) {
+extern "C" int mi_moe_scattered_gemm_ws(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
+                                        const int32_t* expert_offsets, int L, int K, int N, int E, int k,
+                                        int grouped_in, int grouped_out, int dtype, int cfg, void* ws,
+                                        size_t ws_bytes, mi_moe_stream_t stream) {
   int rc = check_common(in, w, out, sorted_scattered, expert_offsets, L, K, N, E, k, dtype,
                         !grouped_in || !grouped_out);
   if (rc != MI_MOE_OK) return rc;
+  if ((rc = check_ws(ws, ws_bytes)) != MI_MOE_OK) return rc;
   GemmArgs a;
   a.in = in; a.w = w; a.out = out;
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = K; a.N = N; a.E = E; a.kdiv = k; a.n_tiles = 0;
-  a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1;
+  a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1; a.ws = ws;
   return run_gemm(a, dtype, false, cfg, L, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int mi_moe_scattered_gemm_wt(const void* in, const void* w_kn, void* out, const int32_t* sorted_scattered,
-                                        const int32_t* expert_offsets, int L, int K, int N, int E, int k,
-                                        int grouped_in, int grouped_out, int dtype, mi_moe_stream_t stream) {
+extern "C" int mi_moe_scattered_gemm_cfg(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
+                                         const int32_t* expert_offsets, int L, int K, int N, int E, int k,
+                                         int grouped_in, int grouped_out, int dtype, int cfg,
+                                         mi_moe_stream_t stream) {
+  return mi_moe_scattered_gemm_ws(in, w, out, sorted_scattered, expert_offsets, L, K, N, E, k, grouped_in,
+                                  grouped_out, dtype, cfg, nullptr, 0, stream);
+}
+
+extern "C" int mi_moe_scattered_gemm_wt_ws(const void* in, const void* w_kn, void* out,
+                                           const int32_t* sorted_scattered, const int32_t* expert_offsets, int L,
+                                           int K, int N, int E, int k, int grouped_in, int grouped_out, int dtype,
+                                           void* ws, size_t ws_bytes, mi_moe_stream_t stream) {
   int rc = check_common(in, w_kn, out, sorted_scattered, expert_offsets, L, K, N, E, k, dtype,
                         !grouped_in || !grouped_out);
   if (rc != MI_MOE_OK) return rc;
   if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if ((rc = check_ws(ws, ws_bytes)) != MI_MOE_OK) return rc;
   if (L == 0) return MI_MOE_OK;
   GemmArgs a;
   a.in = in; a.w = w_kn; a.out = out;
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = K; a.N = N; a.E = E; a.kdiv = k; a.n_tiles = 0;
-  a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1;
+  a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1; a.ws = ws;
   if (!tiled_shape_ok(a, L, false, 2) || !persistent_ok(a)) return MI_MOE_EUNSUPPORTED;
   if (!tiled_aligned(a, 2)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == MI_MOE_BF16) return launch_persistent<bf16_t, 256, 256, 4, 2, false, true>(a, s);
   return launch_persistent<f16_t, 256, 256, 4, 2, false, true>(a, s);
+}
+
+extern "C" int mi_moe_scattered_gemm_wt(const void* in, const void* w_kn, void* out, const int32_t* sorted_scattered,
+                                        const int32_t* expert_offsets, int L, int K, int N, int E, int k,
+                                        int grouped_in, int grouped_out, int dtype, mi_moe_stream_t stream) {
+  return mi_moe_scattered_gemm_wt_ws(in, w_kn, out, sorted_scattered, expert_offsets, L, K, N, E, k, grouped_in,
+                                     grouped_out, dtype, nullptr, 0, stream);
 }
 
 extern "C" int mi_moe_scattered_gemm(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
@@ -1332,17 +1534,25 @@ extern "C" int mi_moe_scattered_gemm(const void* in, const void* w, void* out, c
                                    grouped_out, dtype, -1, stream);
 }
 
-extern "C" int mi_moe_up_swiglu_cfg(const void* x, const void* w_fc, void* act_out, const int32_t* sorted_scattered,
-                                    const int32_t* expert_offsets, int L, int H, int I, int E, int k, int dtype,
-                                    int cfg, mi_moe_stream_t stream) {
+extern "C" int mi_moe_up_swiglu_ws(const void* x, const void* w_fc, void* act_out, const int32_t* sorted_scattered,
+                                   const int32_t* expert_offsets, int L, int H, int I, int E, int k, int dtype,
+                                   int cfg, void* ws, size_t ws_bytes, mi_moe_stream_t stream) {
   int rc = check_common(x, w_fc, act_out, sorted_scattered, expert_offsets, L, H, I, E, k, dtype, true);
   if (rc != MI_MOE_OK) return rc;
+  if ((rc = check_ws(ws, ws_bytes)) != MI_MOE_OK) return rc;
   GemmArgs a;
   a.in = x; a.w = w_fc; a.out = act_out;
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = H; a.N = I; a.E = E; a.kdiv = k; a.n_tiles = 0;
-  a.gather = 1; a.scatter = 0; a.remap = 1;
+  a.gather = 1; a.scatter = 0; a.remap = 1; a.ws = ws;
   return run_gemm(a, dtype, true, cfg, L, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mi_moe_up_swiglu_cfg(const void* x, const void* w_fc, void* act_out, const int32_t* sorted_scattered,
+                                    const int32_t* expert_offsets, int L, int H, int I, int E, int k, int dtype,
+                                    int cfg, mi_moe_stream_t stream) {
+  return mi_moe_up_swiglu_ws(x, w_fc, act_out, sorted_scattered, expert_offsets, L, H, I, E, k, dtype, cfg, nullptr, 0,
+                             stream);
 }
 
 extern "C" int mi_moe_up_swiglu(const void* x, const void* w_fc, void* act_out, const int32_t* sorted_scattered,

@@ -275,10 +275,32 @@ def sort_bin(selected_experts: torch.Tensor, num_experts: int):
 # ------------------------------------------------------------------------------------------------
 
 
+_GEMM_WS: dict = {}
+
+
+def _gemm_workspace(device: torch.device, enabled: bool = True):
+    """(tensor, bytes) of the workspace that lets the persistent grouped GEMM cut the tiles of its last, partly
+    filled round along K (mi_moe_grouped_gemm_workspace_bytes: one fp32 partial tile per CU, 64 MiB on 256 CUs).
+    One per device and stream, kept for the life of the process; its contents carry nothing between calls."""
+    if not enabled:
+        return None, 0
+    key = (device.index, _stream())
+    ws = _GEMM_WS.get(key)
+    if ws is None:
+        n = _lib.load().mi_moe_grouped_gemm_workspace_bytes()
+        if n == 0:
+            return None, 0
+        ws = torch.empty(n, dtype=torch.uint8, device=device)
+        _GEMM_WS[key] = ws
+    return ws, ws.numel()
+
+
 def scattered_gemm(inputs: torch.Tensor, weight: torch.Tensor, k: int, sorted_scattered_idxs: torch.Tensor,
                    expert_offsets: torch.Tensor, grouped_in: bool, grouped_out: bool, cfg: int = -1,
-                   weight_kn: bool = False) -> torch.Tensor:
+                   weight_kn: bool = False, split_k: bool = True) -> torch.Tensor:
     """Grouped GEMM with the weight in native (E, out, in) layout; returns (L, out).
+
+    ``split_k``: hand the persistent kernel its workspace (see _gemm_workspace); False runs every tile whole.
 
     ``weight_kn``: the weight is (E, in, out) instead (``inputs @ weight[e]``, the form of the backward's data
     gradients).  Shapes the transposed-weight kernel does not take are transposed once and run the normal way."""
@@ -301,10 +323,12 @@ def scattered_gemm(inputs: torch.Tensor, weight: torch.Tensor, k: int, sorted_sc
         raise ValueError("scattered inputs must have L / k rows")
     out = torch.empty((L, N), dtype=inputs.dtype, device=inputs.device)
     lib = _lib.load()
+    ws, ws_bytes = _gemm_workspace(inputs.device, split_k)
     if weight_kn:
         with _stage("scattered_gemm"):
-            rc = lib.mi_moe_scattered_gemm_wt(_ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N, E, k,
-                                              int(grouped_in), int(grouped_out), _code(inputs.dtype), _stream())
+            rc = lib.mi_moe_scattered_gemm_wt_ws(_ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N,
+                                                 E, k, int(grouped_in), int(grouped_out), _code(inputs.dtype),
+                                                 _ptr(ws), ws_bytes, _stream())
         if rc == 0:
             return out
         if rc not in (_lib.MI_MOE_EUNSUPPORTED, _lib.MI_MOE_EDTYPE, _lib.MI_MOE_EALIGN):
@@ -314,9 +338,9 @@ def scattered_gemm(inputs: torch.Tensor, weight: torch.Tensor, k: int, sorted_sc
                    "copy of the weights for this call")
         weight = weight.transpose(1, 2).contiguous()
     with _stage("scattered_gemm"):
-        rc = _gemm_or_slow(lambda c: lib.mi_moe_scattered_gemm_cfg(
+        rc = _gemm_or_slow(lambda c: lib.mi_moe_scattered_gemm_ws(
             _ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N, E, k, int(grouped_in),
-            int(grouped_out), _code(inputs.dtype), c, _stream()), cfg, K, N, inputs.dtype)
+            int(grouped_out), _code(inputs.dtype), c, _ptr(ws), ws_bytes, _stream()), cfg, K, N, inputs.dtype)
         check(rc)
     return out
 
@@ -546,8 +570,9 @@ def scattered_experts(inputs: torch.Tensor, expert_weights: torch.Tensor, k: int
 
 
 def up_swiglu(x: torch.Tensor, w_fc: torch.Tensor, k: int, sorted_scattered_idxs: torch.Tensor,
-              expert_offsets: torch.Tensor, cfg: int = -1) -> torch.Tensor:
-    """Up-projection with SwiGLU fused: x (T, H), w_fc (E, 2I, H) -> (L, I) in grouped order."""
+              expert_offsets: torch.Tensor, cfg: int = -1, split_k: bool = True) -> torch.Tensor:
+    """Up-projection with SwiGLU fused: x (T, H), w_fc (E, 2I, H) -> (L, I) in grouped order
+    (``split_k`` as in scattered_gemm)."""
     _dev(x, w_fc, sorted_scattered_idxs, expert_offsets)
     _no_grad(x, w_fc)
     x = x.contiguous()
@@ -562,10 +587,11 @@ def up_swiglu(x: torch.Tensor, w_fc: torch.Tensor, k: int, sorted_scattered_idxs
         raise ValueError("x must have L / k rows")
     act = torch.empty((L, I2 // 2), dtype=x.dtype, device=x.device)
     lib = _lib.load()
+    ws, ws_bytes = _gemm_workspace(x.device, split_k)
     with _stage("up_swiglu"):
-        check(_gemm_or_slow(lambda c: lib.mi_moe_up_swiglu_cfg(
-            _ptr(x), _ptr(w_fc), _ptr(act), _ptr(ss), _ptr(off), L, H, I2 // 2, E, k, _code(x.dtype), c, _stream()),
-            cfg, H, I2 // 2, x.dtype))
+        check(_gemm_or_slow(lambda c: lib.mi_moe_up_swiglu_ws(
+            _ptr(x), _ptr(w_fc), _ptr(act), _ptr(ss), _ptr(off), L, H, I2 // 2, E, k, _code(x.dtype), c, _ptr(ws),
+            ws_bytes, _stream()), cfg, H, I2 // 2, x.dtype))
     return act
 
 

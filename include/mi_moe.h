@@ -191,6 +191,27 @@ int mi_moe_scattered_gemm_cfg(const void* in, const void* w, void* out, const in
                               int grouped_in, int grouped_out, int dtype, int cfg, mi_moe_stream_t stream);
 
 /*
+ * The same three products with a workspace for the persistent tile kernel (cfg 7 / what -1 picks for large expert
+ * loads; no counterpart in the reference, whose kernels launch one workgroup per tile).  That kernel gives every
+ * CU a list of 256 x 256 tiles; when the tiles do not fill the last round, the CUs without a tile wait for one
+ * tile time -- a tenth of the down-projection of a Mixtral-shape layer (4.5 rounds of tiles, each 14336 long).
+ * With a workspace the tiles of that round are cut into 2 .. 4 ranges of K, each range writes an fp32 partial
+ * tile, and a second small launch adds a tile's parts in a fixed order and applies the epilogue: results are
+ * reproducible run to run, and equal to the unsplit kernel's up to the order of the fp32 sums.  Used only where it
+ * pays (K >= 5120 and a last round at most half full); otherwise, and with ws == NULL, the call is exactly the one
+ * without a workspace.  ws: mi_moe_grouped_gemm_workspace_bytes() bytes (one partial tile per CU of the current
+ * device; 0 if there is no device), 16-byte aligned, MI_MOE_EWORKSPACE / MI_MOE_EALIGN otherwise; contents need
+ * no initialisation and carry nothing between calls; calls that overlap in time need separate workspaces.
+ */
+size_t mi_moe_grouped_gemm_workspace_bytes(void);
+int mi_moe_scattered_gemm_ws(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
+                             const int32_t* expert_offsets, int L, int K, int N, int E, int k, int grouped_in,
+                             int grouped_out, int dtype, int cfg, void* ws, size_t ws_bytes, mi_moe_stream_t stream);
+int mi_moe_scattered_gemm_wt_ws(const void* in, const void* w_kn, void* out, const int32_t* sorted_scattered,
+                                const int32_t* expert_offsets, int L, int K, int N, int E, int k, int grouped_in,
+                                int grouped_out, int dtype, void* ws, size_t ws_bytes, mi_moe_stream_t stream);
+
+/*
  * Up-projection with SwiGLU fused into the epilogue:
  *     h = x[sorted_scattered[i] / k] @ w_fc[e_i]^T  (2I wide: rows [0,I) of w_fc are "up", [I,2I) "gate")
  *     act_out[i, :] = h[:I] * silu(h[I:])           (grouped order, `dtype`)
@@ -204,6 +225,10 @@ int mi_moe_up_swiglu(const void* x, const void* w_fc, void* act_out, const int32
 int mi_moe_up_swiglu_cfg(const void* x, const void* w_fc, void* act_out, const int32_t* sorted_scattered,
                          const int32_t* expert_offsets, int L, int H, int I, int E, int k, int dtype, int cfg,
                          mi_moe_stream_t stream);
+/* ... and with the persistent kernel's workspace (see mi_moe_scattered_gemm_ws) */
+int mi_moe_up_swiglu_ws(const void* x, const void* w_fc, void* act_out, const int32_t* sorted_scattered,
+                        const int32_t* expert_offsets, int L, int H, int I, int E, int k, int dtype, int cfg,
+                        void* ws, size_t ws_bytes, mi_moe_stream_t stream);
 
 /*
  * Gate-weighted combine:  y[t, :] = sum_j gates[t, j] * o[t*k + j, :]   (fp32 accumulation).

@@ -98,6 +98,14 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_scattered_gemm(p16, p16, p16, p16, p16, 16, 12, 8, 4, 2, 0, 1, _lib.BF16, None) == E_UNSUP
     assert lib.mi_moe_scattered_gemm(ctypes.c_void_p(4098), p16, p16, p16, p16, 16, 16, 8, 4, 2, 0, 1, _lib.BF16, None) == -4
     assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 16, 0, 8, 4, 2, 0, 1, _lib.BF16, None) == E_SHAPE
+    # the workspace variants: a workspace that is too small (any size is, where no GPU tells the CU count) or
+    # misplaced is refused; no workspace is the call without one
+    need = lib.mi_moe_grouped_gemm_workspace_bytes()
+    assert need == 0 or need % (256 * 256 * 4) == 0
+    assert lib.mi_moe_scattered_gemm_ws(p16, p16, p16, p16, p16, 16, 16, 8, 4, 2, 0, 1, _lib.BF16, -1, p16, 8, None) == E_WS
+    assert lib.mi_moe_up_swiglu_ws(p16, p16, p16, p16, p16, 16, 16, 8, 4, 2, _lib.BF16, -1, p16, 8, None) == E_WS
+    assert lib.mi_moe_scattered_gemm_wt_ws(p16, p16, p16, p16, p16, 16, 16, 8, 4, 2, 0, 1, _lib.BF16, p16, 8, None) == E_WS
+    assert lib.mi_moe_scattered_gemm_ws(p16, p16, p16, p16, p16, 16, 12, 8, 4, 2, 0, 1, _lib.BF16, -1, None, 0, None) == E_UNSUP
     assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 16, 8, 8, 4, 2, 0, 1, 7, None) == E_DTYPE
     assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 16, 8, 8, 4, 2, 0, 1, _lib.BF16, None) == E_NULL
     assert lib.mi_moe_scattered_gemm(None, None, None, None, None, 0, 8, 8, 4, 2, 0, 1, _lib.BF16, None) == 0

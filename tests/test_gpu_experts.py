@@ -10,6 +10,8 @@ import torch
 
 from oracle import moe_oracle as oracle
 
+from _parity import assert_close_scaled
+
 pytestmark = pytest.mark.gpu
 
 TOL = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.bfloat16: dict(rtol=2e-2, atol=2e-2),
@@ -188,6 +190,63 @@ def test_gemm_empty_experts_and_single_expert(device):
         out = ops.scattered_gemm(x.to(device), w.to(device), k, ss.to(device), off.to(device), False, False, cfg=cfg)
         ref = x.float() @ w[9].float().t()
         torch.testing.assert_close(out.cpu().float(), ref, rtol=2e-2, atol=2e-2)
+
+
+# Shapes whose last round of 256 x 256 tiles is partly filled and whose contraction is long enough for the persistent
+# kernel to cut those tiles along K (with 256 CUs: four parts per tile, two parts per tile, one tile per XCD).
+SPLIT_K_CASES = [
+    ("four parts", [5000, 5000, 5000, 5000], 8192, 1024),
+    ("two parts", [7000, 6000, 5200, 5000], 8192, 1024),
+    ("ragged", [1, 9000, 0, 300, 12000, 257], 6144, 768),
+]
+
+
+@pytest.mark.parametrize("form", ["plain", "swiglu", "weight_kn"])
+@pytest.mark.parametrize("name,counts,K,N", SPLIT_K_CASES)
+def test_split_k_of_the_last_round(device, form, name, counts, K, N):
+    """The persistent kernel with its workspace (tiles of the last round cut along K, summed by the finishing
+    launch) against the same kernel without it and against an fp32 product of the same rounded operands:
+    same results up to the order of the fp32 sums, and the same bits from run to run."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(len(counts) * 131 + K)
+    E, L = len(counts), sum(counts)
+    off = torch.tensor(counts).cumsum(0).to(torch.int32).to(device)
+    ss = torch.randperm(L, generator=g).to(torch.int32).to(device)     # scattered output rows
+    inp = (torch.randn(L, K, generator=g) * 0.5).to(torch.bfloat16).to(device)
+    rows_w = 2 * N if form == "swiglu" else N
+    w = (torch.randn(E, rows_w, K, generator=g) * 0.05).to(torch.bfloat16).to(device)
+    w_kn = w.transpose(1, 2).contiguous() if form == "weight_kn" else None
+    print(f"split-K {form} {name}", flush=True)
+
+    def run(split):
+        if form == "swiglu":
+            return ops.up_swiglu(inp, w, 1, torch.arange(L, dtype=torch.int32, device=device), off, cfg=7, split_k=split)
+        if form == "weight_kn":
+            return ops.scattered_gemm(inp, w_kn, 1, ss, off, True, False, weight_kn=True, split_k=split)
+        return ops.scattered_gemm(inp, w, 1, ss, off, True, False, cfg=7, split_k=split)
+
+    whole, split, again = run(False), run(True), run(True)
+    assert torch.equal(split, again), "not reproducible"
+    # fp32 product of the same operands, expert by expert (a library GEMM on the device)
+    ref = torch.empty((L, N), dtype=torch.float32, device=device)
+    prev = 0
+    for e, end in enumerate(off.tolist()):
+        h = inp[prev:end].float() @ w[e].float().t()
+        if form == "swiglu":
+            h = h[:, :N] * torch.nn.functional.silu(h[:, N:])
+        ref[prev:end] = h
+        prev = end
+    if form != "swiglu":
+        scattered = torch.empty_like(ref)
+        scattered[ss.long()] = ref
+        ref = scattered
+    assert_close_scaled(split, ref, torch.bfloat16, rtol=2e-2, atol=2e-2, what=f"split-K {form} {name}")
+    # against the unsplit kernel: the fp32 sums differ in their last bits only, which flips a bf16 rounding now and then
+    differ = (split != whole)
+    assert differ.float().mean().item() < 2e-3
+    # (one bf16 step of the value, or -- for results next to zero -- the reordering error of the fp32 sum itself)
+    one_step = (split.float() - whole.float()).abs() <= whole.float().abs() * 2 ** -7 + 1e-4
+    assert bool(one_step.all())
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
