@@ -344,7 +344,10 @@ def main():
             ((out_ * dy).sum() + 0.01 * get_aux_loss()).backward()
 
         train = {}
-        for name, kernels in (("kernels", True), ("eager", False)):
+        # kernels: the up-projection's pre-activation is kept for the backward (the module's default);
+        # kernels_recompute: it is recomputed there (MoE.keep_preactivation = False)
+        for name, kernels in (("kernels", True), ("kernels_recompute", True), ("eager", False)):
+            m.keep_preactivation = name != "kernels_recompute"
             torch.cuda.reset_peak_memory_stats()
             for _ in range(3):
                 train_step(kernels)

@@ -50,6 +50,7 @@ SIGNATURES: dict[str, tuple] = {
     "mi_moe_combine": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mi_moe_combine_block_tail": (_i, [_vp, _vp, _vp, _vp, ctypes.c_float, _i, _vp, _i, _i, _i, _i, _vp]),
     "mi_moe_swiglu_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "mi_moe_swiglu_forward": (_i, [_vp, _vp, _i, _i, _i, _vp]),
     "mi_moe_combine_grad_gates": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mi_moe_grouped_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mi_moe_grouped_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _vp]),

@@ -8,9 +8,12 @@ gradients (fp32 and odd shapes run a one-thread-per-element form of it; nothing 
 (lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:91-101); this module is the counterpart for the
 gradient, built on this package's forward kernels.
 
-Memory kept for the backward: x, the gates and the routing indices; the (L, 2I) pre-activation is recomputed,
-the (L, I) activation follows from it, and the (L, H) expert outputs are never needed (the gradient of a router
-weight, <dy[t], w_proj[e] a>, is taken as <w_proj[e]^T dy[t], a>).
+Memory kept for the backward: x, the gates, the routing indices and -- by default -- the (L, 2I) pre-activation
+h of the up-projection (the forward then runs the up-projection unfused: grouped GEMM, then the element-wise
+SwiGLU on the stored h, as the reference does, moe.py:273-281); with ``keep_preactivation=False`` h is recomputed
+in the backward from x and the forward keeps its fused up-projection (one more grouped GEMM per step, L * 2I
+elements less memory).  The (L, I) activation follows from h, and the (L, H) expert outputs are never needed (the
+gradient of a router weight, <dy[t], w_proj[e] a>, is taken as <w_proj[e]^T dy[t], a>).
 """
 
 from __future__ import annotations
@@ -24,17 +27,22 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
     """y[t] = sum_j gates[t, j] * ( swiglu(x[t] @ w_fc[e]^T) @ w_proj[e]^T ),  e = expert of slot (t, j)."""
 
     @staticmethod
-    def forward(ctx, x, w_fc, w_proj, gates, sorted_scattered, expert_offsets, k):
-        act = ops.up_swiglu(x, w_fc, k, sorted_scattered, expert_offsets)
+    def forward(ctx, x, w_fc, w_proj, gates, sorted_scattered, expert_offsets, k, keep_preactivation=True):
+        h = None
+        if keep_preactivation:
+            h = ops.scattered_gemm(x, w_fc, k, sorted_scattered, expert_offsets, False, True)
+            act = ops.swiglu_forward(h)
+        else:
+            act = ops.up_swiglu(x, w_fc, k, sorted_scattered, expert_offsets)
         o = ops.scattered_gemm(act, w_proj, 1, sorted_scattered, expert_offsets, True, False)
         y = ops.combine(o, gates)
-        ctx.save_for_backward(x, w_fc, w_proj, gates, sorted_scattered, expert_offsets)
+        ctx.save_for_backward(x, w_fc, w_proj, gates, sorted_scattered, expert_offsets, h)
         ctx.k = k
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        x, w_fc, w_proj, gates, ss, off = ctx.saved_tensors
+        x, w_fc, w_proj, gates, ss, off, h = ctx.saved_tensors
         k = ctx.k
         T, H = x.shape
         E, I2, _ = w_fc.shape
@@ -44,10 +52,11 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
 
         # gradient w.r.t. the SwiGLU output a, in sorted order and before the router weight: dy[t_i] @ w_proj[e_i]
         d_act = ops.scattered_gemm(dy, w_proj, k, ss, off, False, True, weight_kn=True)
-        # pre-activation recomputed; one pass then gives d_h (with the router weight g_i of the row applied),
+        # pre-activation kept or recomputed; one pass then gives d_h (with the router weight g_i of the row applied),
         # g_i * a_i for the down-projection's weight gradient, and the gradient of the router weights,
         # <dy[t], w_proj[e] a_i> = <d_act_i, a_i>
-        h = ops.scattered_gemm(x, w_fc, k, ss, off, False, True)
+        if h is None:
+            h = ops.scattered_gemm(x, w_fc, k, ss, off, False, True)
         if half:
             d_h, act_g, d_gates = ops.swiglu_backward(h, d_act, gates, ss, want_act=True, want_gate_grad=True)
         else:
@@ -74,7 +83,7 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
         tok32 = torch.div(ss, k, rounding_mode="floor").to(torch.int32)
         d_w_fc = ops.grouped_wgrad(d_h, x, off, None, tok32)
         d_w_proj = ops.grouped_wgrad(dy, act_g, off, tok32, None)
-        return dx, d_w_fc, d_w_proj, d_gates, None, None, None
+        return dx, d_w_fc, d_w_proj, d_gates, None, None, None, None
 
 
 class ScatteredExperts(torch.autograd.Function):

@@ -90,6 +90,50 @@ __global__ __launch_bounds__(256) void combine_grad_gates_kernel(const T* __rest
   }
 }
 
+// a = up * silu(gate) from a stored pre-activation h = [up | gate]: the activation of the unfused forward that a
+// training step takes when it keeps h for the backward instead of recomputing it.  fp32 arithmetic on the rounded
+// h, one rounding of the result (what GLUActivation does to the output of the grouped GEMM, activations/glu.py:42-43).
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_forward_kernel(const T* __restrict__ h, T* __restrict__ act, long chunks,
+                                                             int cpr) {
+  // chunk c: row c / cpr, columns 8 * (c % cpr) .. + 8
+  for (long c = (long)blockIdx.x * 256 + threadIdx.x; c < chunks; c += (long)gridDim.x * 256) {
+    const long row = c / cpr;
+    const int col = (int)(c - row * cpr) * 8;
+    const T* hp = h + row * (long)(2 * cpr * 8) + col;
+    const u32x4 up = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(hp));
+    const u32x4 gt = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(hp + cpr * 8));
+    u32x4 out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float u0 = unpack_lo<T>(up[i]), u1 = unpack_hi<T>(up[i]);
+      const float g0 = unpack_lo<T>(gt[i]), g1 = unpack_hi<T>(gt[i]);
+      out[i] = pack2<T>(u0 * silu_f32(g0), u1 * silu_f32(g1));
+    }
+    __builtin_nontemporal_store(out, reinterpret_cast<u32x4*>(act + row * (long)(cpr * 8) + col));
+  }
+}
+
+extern "C" int mi_moe_swiglu_forward(const void* h, void* act_out, int L, int I, int dtype, mi_moe_stream_t stream) {
+  if (L < 0 || I < 1) return MI_MOE_ESHAPE;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (I % 8 != 0) return MI_MOE_EUNSUPPORTED;
+  if (L == 0) return MI_MOE_OK;
+  if (!h || !act_out) return MI_MOE_ENULL;
+  if (!mi_aligned(h, 16) || !mi_aligned(act_out, 16)) return MI_MOE_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const long chunks = (long)L * (I / 8);
+  long blocks = (chunks + 255) / 256;
+  if (blocks > 256L * 32) blocks = 256L * 32;
+  if (dtype == MI_MOE_BF16)
+    hipLaunchKernelGGL((swiglu_forward_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s,
+                       static_cast<const bf16_t*>(h), static_cast<bf16_t*>(act_out), chunks, I / 8);
+  else
+    hipLaunchKernelGGL((swiglu_forward_kernel<f16_t>), dim3((unsigned)blocks), dim3(256), 0, s,
+                       static_cast<const f16_t*>(h), static_cast<f16_t*>(act_out), chunks, I / 8);
+  return mi_launch_status();
+}
+
 extern "C" int mi_moe_swiglu_backward(const void* h, const void* d_act, const void* gates,
                                       const int32_t* sorted_scattered, void* d_h, void* act_g, void* d_gates, int L,
                                       int I, int dtype, mi_moe_stream_t stream) {

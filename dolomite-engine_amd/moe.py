@@ -165,6 +165,9 @@ class MoE(nn.Module):
         self.num_experts = num_experts
         self.top_k = num_experts_per_tok
         self.use_padding_free_transformer = use_padding_free_transformer
+        # training on the kernel branch: keep the (slots, 2 * intermediate) pre-activation of the up-projection for
+        # the backward (faster) or recompute it there (one grouped GEMM more, that much memory less)
+        self.keep_preactivation = True
 
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
@@ -366,7 +369,7 @@ class MoE(nn.Module):
                 assert self.c_fc.bias is None and tail is None
                 hidden_states = ScatteredSwiGLUExperts.apply(
                     hidden_states, self.c_fc.weight, self.c_proj.weight, router_weights, sorted_scattered_idxs,
-                    expert_offsets, self.top_k
+                    expert_offsets, self.top_k, self.keep_preactivation
                 )
             elif self.c_fc.weight_q is not None:
                 if not self._fused_swiglu:

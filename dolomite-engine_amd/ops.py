@@ -390,6 +390,25 @@ def combine(o: torch.Tensor, gates: torch.Tensor, shared: torch.Tensor | None = 
     return y
 
 
+def swiglu_forward(h: torch.Tensor) -> torch.Tensor:
+    """``h[:, :I] * silu(h[:, I:])`` for a stored pre-activation h (L, 2I) (activations/glu.py:42-43): fp32
+    arithmetic on the rounded h, one rounding.  16-bit dtypes with I % 8 == 0 run the kernel, anything else torch."""
+    _dev(h)
+    _no_grad(h)
+    h = h.contiguous()
+    L, I2 = h.shape
+    I = I2 // 2
+    if I2 % 2:
+        raise ValueError("h must be (L, 2I)")
+    if h.dtype not in (torch.float16, torch.bfloat16) or I % 8:
+        up, gate = h[:, :I].float(), h[:, I:].float()
+        return (up * gate * torch.sigmoid(gate)).to(h.dtype)
+    act = torch.empty((L, I), dtype=h.dtype, device=h.device)
+    with _stage("swiglu_forward"):
+        check(_lib.load().mi_moe_swiglu_forward(_ptr(h), _ptr(act), L, I, _code(h.dtype), _stream()))
+    return act
+
+
 def swiglu_backward(h: torch.Tensor, d_act: torch.Tensor, gates: torch.Tensor | None = None,
                     sorted_scattered_idxs: torch.Tensor | None = None, want_act: bool = False,
                     want_gate_grad: bool = False):

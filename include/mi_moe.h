@@ -268,6 +268,11 @@ int mi_moe_combine_block_tail(const void* o, const void* gates, const void* shar
  */
 int mi_moe_swiglu_backward(const void* h, const void* d_act, const void* gates, const int32_t* sorted_scattered,
                            void* d_h, void* act_g, void* d_gates, int L, int I, int dtype, mi_moe_stream_t stream);
+/* The activation on its own, act_out (L, I) = h[:, :I] * silu(h[:, I:]) for a stored pre-activation h (L, 2I):
+ * the GLUActivation the reference applies to the output of the up-projection (moe.py:281, glu.py:42-43).  A
+ * training step that keeps h for the backward uses the unfused pair (mi_moe_scattered_gemm, this) in place of
+ * mi_moe_up_swiglu.  I % 8 == 0. */
+int mi_moe_swiglu_forward(const void* h, void* act_out, int L, int I, int dtype, mi_moe_stream_t stream);
 /* d_gates[t, j] = <dy[t, :], o[t*k + j, :]>: the gradient of mi_moe_combine w.r.t. the gates.  H % 8 == 0. */
 int mi_moe_combine_grad_gates(const void* o, const void* dy, void* d_gates, int T, int k, int H, int dtype,
                               mi_moe_stream_t stream);

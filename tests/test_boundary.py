@@ -90,6 +90,10 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_sort_bin_workspace_bytes(1 << 23, 1000) > (1 << 20)
     assert lib.mi_moe_sort_bin_static(ctypes.c_void_p(256), 1 << 20, 8, 1000, ctypes.c_void_p(256), ctypes.c_void_p(256),
                                       ctypes.c_void_p(256), None) == -7
+    assert lib.mi_moe_swiglu_forward(None, None, 4, 12, _lib.BF16, None) == E_UNSUP
+    assert lib.mi_moe_swiglu_forward(None, None, 4, 16, _lib.F32, None) == E_DTYPE
+    assert lib.mi_moe_swiglu_forward(None, None, 4, 16, _lib.BF16, None) == E_NULL
+    assert lib.mi_moe_swiglu_forward(None, None, 0, 16, _lib.BF16, None) == 0
     assert lib.mi_moe_grouped_wgrad_naive(None, None, None, None, None, None, 16, 8, 8, 4, 7, None) == E_DTYPE
     assert lib.mi_moe_grouped_wgrad_naive(None, None, None, None, None, None, 16, 8, 8, 4, _lib.F32, None) == E_NULL
     # 16-bit problems the matrix-core kernels cannot take are refused, not run on the slow kernel behind the

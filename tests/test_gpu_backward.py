@@ -53,6 +53,22 @@ def test_swiglu_backward(device, dtype, L, I, k, routed):
         assert d_gates is None
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("L,I", [(1, 8), (77, 136), (1000, 512), (5, 100)])
+def test_swiglu_forward(device, dtype, L, I):
+    """a = up * silu(gate) of a stored pre-activation against the closed form in fp64 on the same rounded h
+    (activations/glu.py:42-43); (5, 100) and fp32 take the torch form inside the wrapper."""
+    g = torch.Generator().manual_seed(L + I)
+    h = (torch.randn(L, 2 * I, generator=g) * 2).to(dtype)
+    got = _ops().swiglu_forward(h.to(device))
+    hd = h.double()
+    ref = hd[:, :I] * hd[:, I:] * torch.sigmoid(hd[:, I:])
+    assert got.shape == (L, I) and got.dtype == dtype
+    tol = {torch.float32: 1e-6, torch.float16: 1e-3, torch.bfloat16: 8e-3}[dtype]
+    torch.testing.assert_close(got.cpu().double(), ref, rtol=tol, atol=tol)
+    assert got.abs().max() > 0.5
+
+
 def test_swiglu_backward_empty_and_errors(device):
     ops = _ops()
     out, act_g, d_gates = ops.swiglu_backward(torch.empty(0, 32, device=device, dtype=torch.bfloat16),

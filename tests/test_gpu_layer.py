@@ -331,7 +331,7 @@ def test_low_level_ops_record_no_gradient(device):
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, dict(rtol=2e-3, atol=2e-5)), (torch.bfloat16, dict(rtol=5e-2, atol=2e-2))])
 @pytest.mark.parametrize("shared", [None, 64])
-@pytest.mark.parametrize("activation", ["swiglu", "gelu_pytorch_tanh", "geglu"])
+@pytest.mark.parametrize("activation", ["swiglu", "swiglu-recompute", "gelu_pytorch_tanh", "geglu"])
 def test_training_gradients_match_eager_branch(device, dtype, tol, shared, activation):
     """Training through the kernel branch: output, aux loss and every gradient (input, router, both expert
     weight tensors, shared experts) against torch autograd through the eager branch of the same module.
@@ -340,6 +340,9 @@ def test_training_gradients_match_eager_branch(device, dtype, tol, shared, activ
     from dolomite_engine_amd import Kernel, MoE, enable_kernels
     from dolomite_engine_amd.loss import clear_aux_loss, get_aux_loss
 
+    # "swiglu": the pre-activation of the up-projection is kept for the backward; "swiglu-recompute": recomputed there
+    keep = activation != "swiglu-recompute"
+    activation = activation.split("-")[0]
     if activation != "swiglu" and shared is not None:
         pytest.skip("the shared experts do not depend on the routed experts' activation path")
     torch.manual_seed(21)
@@ -347,6 +350,7 @@ def test_training_gradients_match_eager_branch(device, dtype, tol, shared, activ
             num_experts_per_tok=2, activation_function=activation, add_bias=False, dropout=0.0, init_method="normal",
             initializer_range=0.1, m_width=None, num_layers=1, use_padding_free_transformer=True)
     m = m.to(dtype).to(device).train()
+    m.keep_preactivation = keep
     x0 = torch.randn(300, 128, device=device, dtype=dtype)
     dy = torch.randn(300, 128, device=device, dtype=dtype)
 
