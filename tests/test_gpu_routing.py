@@ -59,7 +59,8 @@ def test_topk_special_values(device):
 
 
 @pytest.mark.parametrize("T,k,E", [(0, 2, 8), (1, 1, 1), (15, 8, 8), (512, 2, 8), (64, 6, 64), (1024, 8, 32),
-                                   (1365, 6, 40), (16384, 8, 32), (32768, 8, 40), (5000, 3, 1000), (4099, 2, 3)])
+                                   (1365, 6, 40), (16384, 8, 32), (32768, 8, 40), (5000, 3, 1000), (4099, 2, 3),
+                                   (70000, 8, 40)])  # the last: more chunks than the launch that fuses passes 2 and 3 takes
 @pytest.mark.parametrize("skew", [False, True])
 def test_sort_bin(device, T, k, E, skew):
     ops = _ops()
