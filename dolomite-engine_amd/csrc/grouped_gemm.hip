@@ -696,23 +696,60 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GemmArgs 
 #define PERSIST_SPLIT_MIN_SLICES 32
 #define PERSIST_WS_TILE_BYTES (256 * 256 * 4)
 
+// Which tiles a workgroup runs.  Workgroup b sits on XCD b % 8 (the hardware deals workgroup ids round-robin to the
+// XCDs) in slot b / 8.  Two ways of dealing the band-ordered tile list to them:
+//   * contiguous (the default): XCD x owns the x-th eighth of the list and deals it to its slots in turn, so the
+//     CUs of an XCD work on neighbouring tiles out of one L2 and an XCD stays with its experts;
+//   * interleaved (PERSIST_REMAP_INTERLEAVE): round r of the whole chip is the tiles [r * grid, (r + 1) * grid), XCD
+//     x taking the x-th run of grid / 8 of them.  All XCDs then work on neighbouring tiles at the same time.  When
+//     an expert has more column tiles than a band is wide (intermediate size 14336: 112 column tiles, bands of 8),
+//     consecutive bands read the same activation rows, and the XCDs share them through the memory-side cache
+//     instead of each fetching them from HBM in its own time: Mixtral-shape layer 5.02 -> 4.73 ms.  With few
+//     column tiles (the band is the whole row) it changes little either way (-1.3 % on the Granite-1B shape,
+//     +1.1 % on the Granite-3B shape), so the host asks for it only from 8 column tiles on.
+// Either way the tiles that do not fill the last round can be cut along K (see PERSIST_SPLIT_MAX).
+#define PERSIST_REMAP_INTERLEAVE 2
+
 struct SplitPlan {
-  int per;          // tiles per XCD (the last XCD may have fewer)
-  int full_rounds;  // rounds in which every slot of the XCD has a tile
-  int rem;          // tiles of the last round
-  int parts;        // K ranges each of them is cut into (1: not split)
+  int base, stride;  // tile of this workgroup in round i < full_rounds: base + i * stride
+  int full_rounds;   // rounds in which every slot has a tile
+  int rem;           // tiles of the last round, the first of them being rem_base
+  int rem_base;
+  int parts;         // K ranges each of them is cut into (1: not split)
+  int lslot;         // this workgroup's slot in the last round: part lslot / rem of tile rem_base + lslot % rem
+  int ws_base;       // first partial-tile slot of the last round's tiles in the workspace
 };
 
-__device__ __forceinline__ SplitPlan persist_split_plan(int total, int xcd, int nslot, int nk, bool have_ws) {
+// xcd / slot of the workgroup (slot < nslot); for the finishing kernel, slot is the tile of the last round it adds up
+__device__ __forceinline__ SplitPlan persist_split_plan(int total, int xcd, int slot, int nslot, int nk, bool have_ws,
+                                                        bool interleave) {
   SplitPlan sp;
-  sp.per = (total + 7) >> 3;
-  int n_x = total - xcd * sp.per;
-  n_x = n_x < 0 ? 0 : (n_x < sp.per ? n_x : sp.per);
-  sp.full_rounds = n_x / nslot;
-  sp.rem = n_x - sp.full_rounds * nslot;
+  int cap;  // slots that share one last round
+  if (interleave) {
+    cap = nslot * 8;
+    sp.lslot = xcd * nslot + slot;
+    sp.base = sp.lslot;
+    sp.stride = cap;
+    sp.full_rounds = total / cap;
+    sp.rem = total - sp.full_rounds * cap;
+    sp.rem_base = sp.full_rounds * cap;
+    sp.ws_base = 0;
+  } else {
+    cap = nslot;
+    const int per = (total + 7) >> 3;
+    int n_x = total - xcd * per;
+    n_x = n_x < 0 ? 0 : (n_x < per ? n_x : per);
+    sp.lslot = slot;
+    sp.base = xcd * per + slot;
+    sp.stride = nslot;
+    sp.full_rounds = n_x / nslot;
+    sp.rem = n_x - sp.full_rounds * nslot;
+    sp.rem_base = xcd * per + sp.full_rounds * nslot;
+    sp.ws_base = xcd * nslot;
+  }
   sp.parts = 1;
   if (have_ws && sp.rem > 0) {
-    int p = nslot / sp.rem;
+    int p = cap / sp.rem;
     if (p > PERSIST_SPLIT_MAX) p = PERSIST_SPLIT_MAX;
     if (p >= 2 && nk / p >= PERSIST_SPLIT_MIN_SLICES && nk - nk / p >= PERSIST_SPLIT_MIN_SAVED) sp.parts = p;
   }
@@ -830,15 +867,16 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   const int total = etab[2 * (a.E - 1)] * a.n_tiles;
   const int xcd = blockIdx.x & 7, slot0 = blockIdx.x >> 3, nslot = gridDim.x >> 3;
   const int nk = a.K / BK;  // >= NSTAGE (host-checked)
-  // this XCD's tiles: full_rounds rounds over all slots, then `rem` tiles, each cut into `parts` K ranges
-  const SplitPlan sp = persist_split_plan(total, xcd, nslot, nk, a.ws != nullptr);
-  const int my_part = sp.parts > 1 ? slot0 / sp.rem : 0, my_rem_tile = sp.rem > 0 ? slot0 % sp.rem : 0;
+  // full_rounds rounds in which every slot has a tile, then `rem` tiles, each cut into `parts` K ranges
+  const SplitPlan sp =
+      persist_split_plan(total, xcd, slot0, nslot, nk, a.ws != nullptr, (a.remap & PERSIST_REMAP_INTERLEAVE) != 0);
+  const int my_part = sp.parts > 1 ? sp.lslot / sp.rem : 0, my_rem_tile = sp.rem > 0 ? sp.lslot % sp.rem : 0;
 
   // i-th tile of this workgroup, or -1
   auto tile_of = [&](int i) -> int {
-    if (i < sp.full_rounds) return xcd * sp.per + slot0 + i * nslot;
-    if (i > sp.full_rounds || slot0 >= sp.rem * sp.parts) return -1;
-    return xcd * sp.per + sp.full_rounds * nslot + my_rem_tile;
+    if (i < sp.full_rounds) return sp.base + i * sp.stride;
+    if (i > sp.full_rounds || sp.lslot >= sp.rem * sp.parts) return -1;
+    return sp.rem_base + my_rem_tile;
   };
   // K slices [k0, k0 + len) of the i-th item
   auto item_k = [&](int i, int& k0, int& len) {
@@ -1103,7 +1141,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     constexpr size_t PART_VECS = (size_t)NB * MB * NW * 64;  // f32x4 per partial tile
     unsigned t = tid;
     asm volatile("" : "+v"(t));  // (keeps the offset from being computed ahead of the tile loop and held through it)
-    f32x4* base = static_cast<f32x4*>(a.ws) + ((size_t)xcd * nslot + (size_t)my_rem_tile * sp.parts + my_part) * PART_VECS;
+    f32x4* base = static_cast<f32x4*>(a.ws) + ((size_t)sp.ws_base + (size_t)my_rem_tile * sp.parts + my_part) * PART_VECS;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -1207,14 +1245,16 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_split_finish_kernel(
   if (wave == 0) persist_expert_table<BM>(a.expert_offsets, a.E, etab);
   __syncthreads();
   const int total = etab[2 * (a.E - 1)] * a.n_tiles;
-  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
-  const SplitPlan sp = persist_split_plan(total, xcd, nslot, a.K / 32, true);
+  // contiguous: workgroup b adds up tile b / 8 of XCD b % 8's last round; interleaved: tile b of the chip's last round
+  const bool interleave = (a.remap & PERSIST_REMAP_INTERLEAVE) != 0;
+  const int xcd = interleave ? 0 : (int)(blockIdx.x & 7), j = interleave ? (int)blockIdx.x : (int)(blockIdx.x >> 3);
+  const SplitPlan sp = persist_split_plan(total, xcd, 0, nslot, a.K / 32, true, interleave);
   if (sp.parts == 1 || j >= sp.rem) return;
   TileCoord tc;
-  persist_locate<BM>(etab, a.E, a.n_tiles, xcd * sp.per + sp.full_rounds * nslot + j, tc);
+  persist_locate<BM>(etab, a.E, a.n_tiles, sp.rem_base + j, tc);
 
   // vector j of thread t of a part lies at [j][t]
-  const f32x4* part = static_cast<const f32x4*>(a.ws) + ((size_t)xcd * nslot + (size_t)j * sp.parts) * PART_VECS + tid;
+  const f32x4* part = static_cast<const f32x4*>(a.ws) + ((size_t)sp.ws_base + (size_t)j * sp.parts) * PART_VECS + tid;
   f32x4 sum[NB][MB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb)
@@ -1343,6 +1383,7 @@ static int launch_persistent(GemmArgs a, hipStream_t s) {
   int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok);
   if (rc != MI_MOE_OK) return rc;
   a.n_tiles = mi_ceil_div(a.N, BN);
+  if (a.n_tiles >= 8) a.remap |= PERSIST_REMAP_INTERLEAVE;  // (see PERSIST_REMAP_INTERLEAVE)
   int cus = 0;
   if ((rc = mi_cu_count(&cus)) != MI_MOE_OK) return rc;
   long max_tiles = ((long)a.L / BM + (a.E < a.L ? a.E : a.L)) * a.n_tiles;

@@ -193,11 +193,13 @@ def test_gemm_empty_experts_and_single_expert(device):
 
 
 # Shapes whose last round of 256 x 256 tiles is partly filled and whose contraction is long enough for the persistent
-# kernel to cut those tiles along K (with 256 CUs: four parts per tile, two parts per tile, one tile per XCD).
+# kernel to cut those tiles along K (with 256 CUs: four parts per tile, two parts per tile, one tile per XCD, and
+# the chip-wide last round of the interleaved tile order).
 SPLIT_K_CASES = [
     ("four parts", [5000, 5000, 5000, 5000], 8192, 1024),
     ("two parts", [7000, 6000, 5200, 5000], 8192, 1024),
     ("ragged", [1, 9000, 0, 300, 12000, 257], 6144, 768),
+    ("eight column tiles", [3000, 2500, 2000, 1500], 8192, 2048),  # the tile order that interleaves the XCDs
 ]
 
 
