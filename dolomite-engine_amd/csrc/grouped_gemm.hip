@@ -1396,9 +1396,10 @@ static int launch_persistent(GemmArgs a, hipStream_t s) {
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, a);
   if ((rc = mi_launch_status()) != MI_MOE_OK || a.ws == nullptr) return rc;
-  // the tiles that were cut: at most half of an XCD's slots hold tiles of a split round
+  // the tiles that were cut: at most half of the slots of a round that was split hold tiles (rounded up: an odd
+  // number of slots per XCD)
   const int nslot = (int)(grid / 8);
-  hipLaunchKernelGGL((grouped_gemm_split_finish_kernel<T, BM, BNW, WM, WN, GLU>), dim3(8u * (unsigned)(nslot / 2)),
+  hipLaunchKernelGGL((grouped_gemm_split_finish_kernel<T, BM, BNW, WM, WN, GLU>), dim3(8u * (unsigned)((nslot + 1) / 2)),
                      dim3(NW * 64), 0, s, a, nslot);
   return mi_launch_status();
 }

@@ -251,6 +251,66 @@ def test_split_k_of_the_last_round(device, form, name, counts, K, N):
     assert bool(one_step.all())
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+def test_persistent_kernel_random_shapes(device, seed):
+    """The persistent kernel's scheduling (tile order by XCD in both forms, last round cut along K, finishing
+    launch, grids smaller than the chip) on random shapes: expert counts from 1 to 130 with empty experts, row
+    counts around the tile edge and up to 66000, contraction lengths from 128 to 8192, 1 to 10 column tiles,
+    all three forms -- against an fp32 product of the same rounded operands."""
+    import random
+
+    ops = _ops()
+    rnd = random.Random(seed)
+    # one shape that once lost tiles: 20 tiles on a grid of 40 (an odd number of slots per XCD), cut in two along K
+    fixed = [(3, 256, 8192, 2400, "plain", [128, 0, 128])] if seed == 2 else []
+    for case in range(24):
+        fixed_counts = None
+        if case < len(fixed):
+            E, L, K, N, form, fixed_counts = fixed[case]
+        else:
+            E = rnd.choice([1, 2, 3, 8, 40, 64, 65, 130])
+            K = 32 * rnd.choice([4, 5, 16, 33, 48, 128, 160, 192, 256])
+            form = rnd.choice(["plain", "plain", "swiglu", "weight_kn"])
+            N = 8 * rnd.choice([1, 16, 31, 32, 64, 96, 128, 256, 300])
+            L = rnd.choice([1, 255, 256, 257, 3000, 10000, 30000, 66000])
+        rows_w = 2 * N if form == "swiglu" else N
+        if L * K * 2 > 1.2e9 or E * rows_w * K * 2 > 1.5e9:
+            continue
+        g = torch.Generator().manual_seed(seed * 100003 + case)
+        p = torch.rand(E, generator=g).pow(rnd.choice([0.5, 3.0, 6.0]))
+        if E > 2:
+            p[torch.rand(E, generator=g) < 0.2] = 0
+        if p.sum() == 0:
+            p[0] = 1
+        counts = torch.bincount(torch.multinomial(p.double(), L, replacement=True, generator=g), minlength=E)
+        if fixed_counts is not None:
+            counts = torch.tensor(fixed_counts)
+        off = counts.cumsum(0).to(torch.int32).to(device)
+        ss = torch.randperm(L, generator=g).to(torch.int32).to(device)
+        inp = (torch.randn(L, K, generator=g) * 0.5).to(torch.bfloat16).to(device)
+        w = (torch.randn(E, rows_w, K, generator=g) * (2.0 / K ** 0.5)).to(torch.bfloat16).to(device)
+        print(f"persistent kernel seed {seed} case {case}: E={E} L={L} K={K} N={N} {form}", flush=True)
+        if form == "swiglu":
+            out = ops.up_swiglu(inp, w, 1, torch.arange(L, dtype=torch.int32, device=device), off, cfg=7)
+        elif form == "weight_kn":
+            out = ops.scattered_gemm(inp, w.transpose(1, 2).contiguous(), 1, ss, off, True, False, weight_kn=True)
+        else:
+            out = ops.scattered_gemm(inp, w, 1, ss, off, True, False, cfg=7)
+        ref = torch.zeros((L, N), dtype=torch.float32, device=device)
+        prev = 0
+        for e, end in enumerate(off.tolist()):
+            if end > prev:
+                h = inp[prev:end].float() @ w[e].float().t()
+                ref[prev:end] = h[:, :N] * torch.nn.functional.silu(h[:, N:]) if form == "swiglu" else h
+            prev = end
+        if form != "swiglu":
+            scattered = torch.empty_like(ref)
+            scattered[ss.long()] = ref
+            ref = scattered
+        err = (out.float() - ref).abs().max().item()
+        assert err <= 1e-2 * ref.abs().max().item() + 1e-3, (case, E, L, K, N, form, err)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,k,H", [(1, 1, 8), (15, 8, 32), (512, 2, 256), (100, 6, 4096), (77, 3, 100), (300, 8, 1536)])
 def test_combine(device, dtype, T, k, H):
