@@ -7,6 +7,15 @@
 // lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:91-101 (call sites moe.py:273-290) and for
 // GLUActivation (activations/glu.py:42-43) when fused.
 //
+// Kernels in this file, in order:
+//   grouped_gemm_kernel             register-staged tiles (any K that is a multiple of one 16-byte chunk; bf16, fp16
+//                                   and fp32): the design notes below
+//   grouped_gemm_dma_kernel         the same tile with the operands brought to LDS by DMA, one tile per workgroup
+//   grouped_gemm_persistent_kernel  one workgroup per CU walking a list of 256 x 256 tiles, two wave groups in
+//                                   ping-pong (large expert loads; its notes stand in front of it), with
+//   grouped_gemm_split_finish_kernel  for the tiles of a last round that were cut along K
+//   grouped_gemm_naive_kernel       one thread per output element, only on request (cfg 3)
+//
 // Design
 //   * One workgroup computes a BM x BN output tile of ONE expert.  The tile list is not built on the
 //     host (that would need the per-expert counts, i.e. a device->host sync): every workgroup derives
