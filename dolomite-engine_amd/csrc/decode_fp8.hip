@@ -321,21 +321,27 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
       for (int m = 0; m < NM; ++m)
         xb[m] = __builtin_bit_cast(frag_t,
                                    *reinterpret_cast<const u32x4*>(xs + xr * (KCH * 2) + (((q * NM + m) ^ dec_xswz(xr)) * 16)));
+      // the whole stage goes to registers first, so that its slot can be refilled before the arithmetic
+      u32x4 wv[2][NM / 2];
 #pragma unroll
       for (int b = 0; b < 2; ++b) {
         const int t = 16 * b + r;
 #pragma unroll
-        for (int h = 0; h < NM / 2; ++h) {
-          const u32x4 wv =
-              *reinterpret_cast<const u32x4*>(ws + t * KCH + (((q * (NM / 2) + h) ^ dec_wswz(t)) * 16));
-          acc[b] = Mfma16<T>::run(Mfma16<T>::widen(wv[0], wv[1]), xb[2 * h], acc[b]);
-          acc[b] = Mfma16<T>::run(Mfma16<T>::widen(wv[2], wv[3]), xb[2 * h + 1], acc[b]);
-        }
+        for (int h = 0; h < NM / 2; ++h)
+          wv[b][h] = *reinterpret_cast<const u32x4*>(ws + t * KCH + (((q * (NM / 2) + h) ^ dec_wswz(t)) * 16));
       }
       asm volatile("" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_waitcnt(dec_waitcnt(63, 0));                // my reads of this slot are done
       dma_stage(i + NS, slot);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int h = 0; h < NM / 2; ++h) {
+          acc[b] = Mfma16<T>::run(Mfma16<T>::widen(wv[b][h][0], wv[b][h][1]), xb[2 * h], acc[b]);
+          acc[b] = Mfma16<T>::run(Mfma16<T>::widen(wv[b][h][2], wv[b][h][3]), xb[2 * h + 1], acc[b]);
+        }
       slot = slot + 1 == NS ? 0 : slot + 1;
     }
     __builtin_amdgcn_s_waitcnt(dec_waitcnt(0, 0));
