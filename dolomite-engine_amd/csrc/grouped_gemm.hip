@@ -718,6 +718,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GemmArgs 
 //     +1.1 % on the Granite-3B shape), so the host asks for it only from 8 column tiles on.
 // Either way the tiles that do not fill the last round can be cut along K (see PERSIST_SPLIT_MAX).
 #define PERSIST_REMAP_INTERLEAVE 2
+#define PERSIST_REMAP_FIXED 4  // the caller chose the form (cfg 8 / 9): the host does not apply its own rule
 
 struct SplitPlan {
   int base, stride;  // tile of this workgroup in round i < full_rounds: base + i * stride
@@ -1392,7 +1393,7 @@ static int launch_persistent(GemmArgs a, hipStream_t s) {
   int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok);
   if (rc != MI_MOE_OK) return rc;
   a.n_tiles = mi_ceil_div(a.N, BN);
-  if (a.n_tiles >= 8) a.remap |= PERSIST_REMAP_INTERLEAVE;  // (see PERSIST_REMAP_INTERLEAVE)
+  if (!(a.remap & PERSIST_REMAP_FIXED) && a.n_tiles >= 8) a.remap |= PERSIST_REMAP_INTERLEAVE;  // (see there)
   int cus = 0;
   if ((rc = mi_cu_count(&cus)) != MI_MOE_OK) return rc;
   long max_tiles = ((long)a.L / BM + (a.E < a.L ? a.E : a.L)) * a.n_tiles;
@@ -1452,6 +1453,12 @@ static int dispatch_cfg(GemmArgs a, int cfg, hipStream_t s) {
     case 2: return launch_tiled<T, 32, 256, 1, 4, GLU>(a, s);
     case 4: return a.K % 32 == 0 ? launch_dma<T, 128, 128, 2, 2, GLU>(a, s) : MI_MOE_EUNSUPPORTED;
     case 7: return persistent_ok(a) ? launch_persistent<T, 256, 256, 4, 2, GLU>(a, s) : MI_MOE_EUNSUPPORTED;
+    case 8:  // the persistent kernel with the tile order fixed: XCDs own contiguous ranges ...
+      a.remap |= PERSIST_REMAP_FIXED;
+      return persistent_ok(a) ? launch_persistent<T, 256, 256, 4, 2, GLU>(a, s) : MI_MOE_EUNSUPPORTED;
+    case 9:  // ... or take consecutive blocks of one chip-wide round
+      a.remap |= PERSIST_REMAP_FIXED | PERSIST_REMAP_INTERLEAVE;
+      return persistent_ok(a) ? launch_persistent<T, 256, 256, 4, 2, GLU>(a, s) : MI_MOE_EUNSUPPORTED;
     default: return MI_MOE_EUNSUPPORTED;
   }
 }

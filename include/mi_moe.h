@@ -184,8 +184,10 @@ int mi_moe_scattered_gemm_wt(const void* in, const void* w_kn, void* out, const 
  * 3 = one thread per output element (any shape); 4 = DMA-staged 128x128 (K % 32 == 0); 7 = persistent
  * DMA-staged 256x256 tiles with 32-wide K slices and the two wave groups of a SIMD alternating between
  * LDS/DMA work and matrix instructions (K % 32 == 0, K >= 128, N % 8 == 0, E <= 256; what -1 picks for
- * large expert loads); 4 and 7 are F16 / BF16 only.  A configuration that does not take the shape or type
- * returns MI_MOE_EUNSUPPORTED. */
+ * large expert loads); 8 / 9 = 7 with the order in which the XCDs take the tiles fixed to "each XCD a contiguous
+ * eighth of the tile list" / "consecutive 32-tile blocks of one chip-wide round" (7 picks the second from 8 column
+ * tiles on; same results either way); 4 and 7 .. 9 are F16 / BF16 only.  A configuration that does not take the
+ * shape or type returns MI_MOE_EUNSUPPORTED. */
 int mi_moe_scattered_gemm_cfg(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
                               const int32_t* expert_offsets, int L, int K, int N, int E, int k,
                               int grouped_in, int grouped_out, int dtype, int cfg, mi_moe_stream_t stream);
