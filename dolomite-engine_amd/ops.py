@@ -290,6 +290,8 @@ def _gemm_workspace(device: torch.device, enabled: bool = True):
         n = _lib.load().mi_moe_grouped_gemm_workspace_bytes()
         if n == 0:
             return None, 0
+        if len(_GEMM_WS) >= 16:  # streams come and go (graph captures): do not keep a buffer for each for ever
+            _GEMM_WS.clear()
         ws = torch.empty(n, dtype=torch.uint8, device=device)
         _GEMM_WS[key] = ws
     return ws, ws.numel()
