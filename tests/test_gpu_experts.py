@@ -400,6 +400,44 @@ def test_fp8_tiled_layout_is_bit_identical(device, T, E, k, H, I):
             ops.fp8_tile(w_pj_q, glu=False)
 
 
+@pytest.mark.parametrize("T,E,k,H,I,skew", [(100, 64, 2, 1024, 512, True), (8, 4, 1, 512, 384, False),
+                                            (37, 16, 3, 2048, 640, True), (9, 40, 1, 384, 1024, False),
+                                            (250, 130, 4, 512, 384, True)])
+def test_fp8_few_rows_per_expert(device, T, E, k, H, I, skew):
+    """The decode regime (at most 8 rows per expert on average) with skewed routing: experts with many times 8
+    rows (several passes of the streaming kernel over one unit) next to experts without any; the smallest case
+    has exactly 8 slots.  Tiled weights must give the bits of the row-major weights where both run the same
+    arithmetic (K >= 512), and both must match the oracle."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(T * 7 + E)
+    se, ss, off = _routing(T, E, k, seed=T + E, skew=skew)
+    counts = torch.diff(off, prepend=torch.zeros(1, dtype=off.dtype))
+    assert T * k <= 8 * E and T * k >= 8
+    if skew:
+        assert counts.max().item() > 16 and counts.min().item() == 0
+    x = _rand((T, H), 1.0, torch.bfloat16, g)
+    w_fc_q, fc_scale = oracle.quantize_fp8_per_channel(torch.randn(E, 2 * I, H, generator=g) * 0.02)
+    w_pj_q, pj_scale = oracle.quantize_fp8_per_channel(torch.randn(E, H, I, generator=g) * 0.02)
+    print(f"fp8 few rows T={T} E={E} k={k} H={H} I={I} max rows {counts.max().item()}", flush=True)
+    xd, ssd, offd = x.to(device), ss.to(device), off.to(device)
+    fc_d, fcs_d, pj_d, pjs_d = (t.to(device) for t in (w_fc_q, fc_scale, w_pj_q, pj_scale))
+    act_t = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd)
+    act_r = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd)
+    if H >= 512:
+        assert torch.equal(act_t, act_r)
+    ref_act = oracle.swiglu(oracle.scattered_experts_oracle(x, oracle.dequant_fp8(w_fc_q, fc_scale), k, se, ss, off,
+                                                            grouped_out=True))
+    torch.testing.assert_close(act_t.cpu().float(), ref_act, rtol=2e-2, atol=2e-3)
+    o_t = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd)
+    o_r = ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd)
+    if I >= 512:
+        assert torch.equal(o_t, o_r)
+    ref_o = oracle.scattered_experts_oracle(act_t.cpu(), oracle.dequant_fp8(w_pj_q, pj_scale), 1, se, ss, off,
+                                            grouped_in=True)
+    torch.testing.assert_close(o_t.cpu().float(), ref_o, rtol=2e-2, atol=2e-3)
+    torch.testing.assert_close(o_r.cpu().float(), ref_o, rtol=2e-2, atol=2e-3)
+
+
 def test_fp8_all_bit_patterns(device):
     """Every e4m3fn byte value is widened exactly: K=256 one-hot activations read out each pattern."""
     ops = _ops()
