@@ -310,13 +310,33 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
                                          (lds_ptr_t)(dst + W_BYTES + j * 1024), 16, 0, 0);
     };
 
+    // What the epilogue needs from memory -- this lane's output row and channel scales -- is requested first, ahead
+    // of the ring's DMA: by the end of the pass it has long arrived, and the pass does not end on a load's latency.
+    // (Being the oldest requests of the wave, they also retire first: the ring's counted waits stay as they are.)
+    const bool store_lane = r < XT && g0 + r < row_end;
+    int orow = g0 + r;
+    f32x4 sc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};   // SwiGLU: up / gate; else: channel blocks 0 / 1
+    if (store_lane) {
+      if (a.scatter) orow = a.sorted_scattered[g0 + r];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int col = GLU ? n0 + 4 * q : n0 + 16 * b + 4 * q;
+        if (col < a.N)
+          sc[b] = *reinterpret_cast<const f32x4*>(a.scale + (size_t)expert * WR * a.N + (GLU ? b * a.N : 0) + col);
+      }
+    }
+
     f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
     const int xr = r & (XT - 1);                             // XT = 8: columns 8..15 mirror 0..7
 #pragma unroll
     for (int p = 0; p < NS; ++p) dma_stage(p, p);
     int slot = 0;
-    for (int i = 0; i < nst; ++i) {
-      __builtin_amdgcn_s_waitcnt(dec_waitcnt((NS - 1) * NDMA, 15));  // stage i has landed
+    // stage i: wait until at most VM younger DMA instructions are in flight, move the stage to registers, refill
+    // its slot (ISSUE) and run the matrix instructions
+    auto step = [&](auto vm_tag, auto issue_tag, int i) {
+      constexpr int VM = decltype(vm_tag)::value;
+      constexpr bool ISSUE = decltype(issue_tag)::value != 0;
+      __builtin_amdgcn_s_waitcnt(dec_waitcnt(VM, 15));               // stage i has landed
       asm volatile("" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
       const unsigned char* ws = ring + slot * STAGE;
@@ -338,7 +358,7 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
       asm volatile("" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_waitcnt(dec_waitcnt(63, 0));                // my reads of this slot are done
-      dma_stage(i + NS, slot);
+      if (ISSUE) dma_stage(i + NS, slot);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int b = 0; b < 2; ++b)
@@ -348,21 +368,28 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
           acc[b] = Mfma16<T>::run(Mfma16<T>::widen(wv[b][h][2], wv[b][h][3]), xb[2 * h + 1], acc[b]);
         }
       slot = slot + 1 == NS ? 0 : slot + 1;
+    };
+    static_assert(NS == 2 || NS == 3, "the unrolled tail below");
+    if (nst >= NS) {
+      for (int i = 0; i < nst - NS; ++i) step(dec_int<(NS - 1) * NDMA>{}, dec_int<1>{}, i);
+      // the last NS stages are all requested: nothing is issued any more and the waits count down
+      if constexpr (NS == 3) step(dec_int<2 * NDMA>{}, dec_int<0>{}, 0);
+      step(dec_int<NDMA>{}, dec_int<0>{}, 0);
+      step(dec_int<0>{}, dec_int<0>{}, 0);
+    } else {
+      // fewer stages than the ring has slots: the prologue's surplus requests re-fetched the last stage
+      for (int i = 0; i < nst; ++i) step(dec_int<(NS - 1) * NDMA>{}, dec_int<1>{}, i);
+      __builtin_amdgcn_s_waitcnt(dec_waitcnt(0, 0));                 // surplus DMA must not outlive the wave's LDS
     }
-    __builtin_amdgcn_s_waitcnt(dec_waitcnt(0, 0));
 
     // acc[b][i]: weight row 16b + 4q + i of this wave, activation row g0 + r
-    if (r < XT && g0 + r < row_end) {
-      const int orow = a.scatter ? a.sorted_scattered[g0 + r] : g0 + r;
+    if (store_lane) {
       if (GLU) {
         const int col = n0 + 4 * q;
         if (col < a.N) {
-          const float* sp = a.scale + (size_t)expert * WR * a.N + col;
-          const f32x4 scu = *reinterpret_cast<const f32x4*>(sp);
-          const f32x4 scg = *reinterpret_cast<const f32x4*>(sp + a.N);
           float v[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) v[i] = (acc[0][i] * scu[i]) * silu_f32(acc[1][i] * scg[i]);
+          for (int i = 0; i < 4; ++i) v[i] = (acc[0][i] * sc[0][i]) * silu_f32(acc[1][i] * sc[1][i]);
           const u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
           *reinterpret_cast<u32x2*>(out + (size_t)orow * a.N + col) = p;
         }
@@ -371,9 +398,8 @@ __global__ __launch_bounds__(256) void decode_fp8_stream_kernel(DecodeArgs a) {
         for (int b = 0; b < 2; ++b) {
           const int col = n0 + 16 * b + 4 * q;
           if (col < a.N) {
-            const f32x4 sc = *reinterpret_cast<const f32x4*>(a.scale + (size_t)expert * a.N + col);
-            const u32x2 p = {pack2<T>(acc[b][0] * sc[0], acc[b][1] * sc[1]),
-                             pack2<T>(acc[b][2] * sc[2], acc[b][3] * sc[3])};
+            const u32x2 p = {pack2<T>(acc[b][0] * sc[b][0], acc[b][1] * sc[b][1]),
+                             pack2<T>(acc[b][2] * sc[b][2], acc[b][3] * sc[b][3])};
             *reinterpret_cast<u32x2*>(out + (size_t)orow * a.N + col) = p;
           }
         }
