@@ -185,9 +185,8 @@ __global__ __launch_bounds__(256) void decode_fp8_kernel(DecodeArgs a) {
 //   activations: an expert with at most 8 rows (the decode case) runs one pass with XT = 8 and a
 //                three-stage ring (MFMA columns 8..15 mirror 0..7 and are never stored); more rows run
 //                passes of 16 with a two-stage ring.  Only ceil(rows/4)*4 rows are fetched.
-// Measured against an empty kernel that merely streams the same rows (no LDS reads, no MFMA) this kernel
-// is within ~10 %: at this size (0.4 - 0.7 GB per launch) launch ramp and tail, not the inner loop,
-// separate it from the 7.3 TB/s a long-running stream reaches on this part.
+// Measured against an empty kernel that merely streams the same bytes through the same ring (no LDS reads,
+// no MFMA; 6.7 - 6.8 TB/s with non-temporal DMA) this kernel is within 5 - 10 %.
 // Needs K % 128 == 0; other shapes take the kernel above.
 // ------------------------------------------------------------------------------------------------
 
