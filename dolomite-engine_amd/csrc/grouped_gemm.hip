@@ -1131,7 +1131,16 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
           const int r = it * RPP + lane / EPI_CPR;
           const u32x4 val = *reinterpret_cast<const u32x4*>(scratch + r * (EPI_COLS * 2) + ((cchunk ^ swz(r)) * 16));
           const int row = tc.row_begin + wm * WTM + mp * 32 + r;
-          if (row < tc.row_end && col < a.N) *reinterpret_cast<u32x4*>(out + (size_t)orow_of[mp][it] * a.N + col) = val;
+          if (row < tc.row_end && col < a.N) {
+            u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)orow_of[mp][it] * a.N + col);
+            // The plain form's output -- the (slots, hidden) rows the combine streams once -- is stored
+            // non-temporal, so that it does not push the operands out of the caches: down-projection of the
+            // 16384-token, 32-expert shape 0.169 -> 0.146 ms (its combine 0.048 -> 0.053 ms); little either way
+            // on the other shapes.  The SwiGLU form's output is the next GEMM's operand and stays cached
+            // (non-temporal there: that GEMM 0.147 -> 0.158 ms).
+            if (!GLU) __builtin_nontemporal_store(val, dst);
+            else *dst = val;
+          }
         }
       }
     }
