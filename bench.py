@@ -143,6 +143,16 @@ def measure_compact(name, device, steps=20, warmup=5):
         for _ in range(warmup):
             m(x)
         torch.cuda.synchronize()
+        # The GPU has been idle (CPU baseline, set-up of this workload) and a 0.1 - 0.5 ms step does not bring its
+        # clocks back up within five steps: warm up for at least 50 ms and time at least 30 ms.
+        t0 = time.perf_counter()
+        m(x)
+        torch.cuda.synchronize()
+        est = max(time.perf_counter() - t0, 1e-5)
+        for _ in range(int(0.05 / est) + 1):
+            m(x)
+        torch.cuda.synchronize()
+        steps = max(steps, int(0.03 / est) + 1)
         t0 = time.perf_counter()
         for _ in range(steps):
             m(x)
