@@ -94,6 +94,7 @@ struct GemmArgs {
   int scatter;  // output row of sorted row i is sorted_scattered[i] (else i)
   int remap;    // XCD-aware tile order
   void* ws;     // persistent kernel: workspace for splitting the last round of tiles along K (or null)
+  int out_nt;   // persistent kernel: store the output non-temporal (set in run_gemm)
 };
 
 
@@ -1133,13 +1134,13 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
           const int row = tc.row_begin + wm * WTM + mp * 32 + r;
           if (row < tc.row_end && col < a.N) {
             u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)orow_of[mp][it] * a.N + col);
-            // The plain form's output -- the (slots, hidden) rows the combine streams once -- is stored
-            // non-temporal, so that it does not push the operands out of the caches: down-projection of the
-            // 16384-token, 32-expert shape 0.169 -> 0.146 ms (its combine 0.048 -> 0.053 ms); little either way
-            // on the other shapes.  The SwiGLU form's output is the next GEMM's operand and stays cached
-            // (non-temporal there: that GEMM 0.147 -> 0.158 ms).
-            if (!GLU) __builtin_nontemporal_store(val, dst);
-            else *dst = val;
+            if (a.out_nt) {  // see persistent_out_nt
+              asm volatile("" ::: "memory");  // (the fences keep the compiler from merging the two stores into
+              __builtin_nontemporal_store(val, dst);  //  one plain store, hoisted or sunk out of the branch)
+              asm volatile("" ::: "memory");
+            } else {
+              *dst = val;
+            }
           }
         }
       }
@@ -1506,7 +1507,20 @@ static int pick_cfg(const GemmArgs& a) {
 // cfg < 0 picks a matrix-core kernel from the shape.  Nothing drops to the one-thread-per-output kernel on its own:
 // a problem the matrix-core kernels cannot take is refused (MI_MOE_EALIGN for a misaligned pointer,
 // MI_MOE_EUNSUPPORTED for the shape) and the caller asks for cfg 3 explicitly if it wants the slow kernel.
+// Cache policy of the persistent kernel's output stores.  The plain form's output -- the (slots, hidden) rows the
+// combine streams once -- is stored non-temporal, so that it does not push the operands out of the caches:
+// down-projection of the 16384-token, 32-expert shape 0.169 -> 0.146 ms (its combine 0.048 -> 0.053 ms), little
+// either way on the other shapes.  The SwiGLU form's output is the next GEMM's operand: up to about the size the
+// memory-side cache can hold next to the weights it stays cached (134 MB on that shape: non-temporal stores would
+// make the GEMM that reads it back 8 % slower); beyond that it would not survive until it is read and only evicts
+// the operands on its way (268 MB on the 32768-token, 40-expert shape: both GEMMs 1 % faster non-temporal).
+static int persistent_out_nt(const GemmArgs& a, bool glu, int elt) {
+  if (!glu) return 1;
+  return (double)a.L * a.N * elt > 192.0 * 1024 * 1024;
+}
+
 static int run_gemm(GemmArgs a, int dtype, bool glu, int cfg, int in_rows_bound, hipStream_t s) {
+  a.out_nt = persistent_out_nt(a, glu, dtype == MI_MOE_F32 ? 4 : 2);
   if (a.L == 0) return MI_MOE_OK;
   if (dtype != MI_MOE_F32 && dtype != MI_MOE_F16 && dtype != MI_MOE_BF16) return MI_MOE_EDTYPE;
   if (cfg == 3) {
@@ -1580,6 +1594,7 @@ extern "C" int mi_moe_scattered_gemm_wt_ws(const void* in, const void* w_kn, voi
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = K; a.N = N; a.E = E; a.kdiv = k; a.n_tiles = 0;
   a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1; a.ws = ws;
+  a.out_nt = persistent_out_nt(a, false, 2);
   if (!tiled_shape_ok(a, L, false, 2) || !persistent_ok(a)) return MI_MOE_EUNSUPPORTED;
   if (!tiled_aligned(a, 2)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
