@@ -246,13 +246,11 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
     const int kpos = step * 64 + q * 16;
     dst[0] = dst[1] = (u32x4){0u, 0u, 0u, 0u};
     if (step < nsteps && kpos < H) {  // the MFMA runs on all lanes: out-of-range k contributes zeros
-      if (NORM) {  // read twice: keep the lines in L2
-        dst[0] = *reinterpret_cast<const u32x4*>(xrow + kpos);
-        dst[1] = *reinterpret_cast<const u32x4*>(xrow + kpos + 8);
-      } else {
-        dst[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xrow + kpos));
-        dst[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xrow + kpos + 8));
-      }
+      // Ordinary (cached) loads: with the norm the rows are read twice, and without it they are read again right
+      // after, as the gathered operand of the up-projection -- which runs 1 - 1.5 % faster on rows this pass left in
+      // the caches than on rows streamed through with the non-temporal policy (and this kernel is no slower).
+      dst[0] = *reinterpret_cast<const u32x4*>(xrow + kpos);
+      dst[1] = *reinterpret_cast<const u32x4*>(xrow + kpos + 8);
     }
   };
   auto open_group = [&](int g) {
