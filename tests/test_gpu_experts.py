@@ -462,3 +462,47 @@ def test_fp8_all_bit_patterns(device):
         want = codes[base:base + T].view(torch.float8_e4m3fn).float()
         want = torch.where(finite[base:base + T], want, torch.zeros_like(want))
         assert torch.equal(got, want.to(torch.bfloat16).float()), f"codes {base}..{base + T}"
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_fp8_random_shapes(device, seed):
+    """The fp8 kernels on random shapes and routings: 1 to 257 tokens, 1 to 64 experts (some without rows, some with
+    many times 8), hidden and intermediate sizes from 128 to 2048 in steps of 128 (one to sixteen ring stages, so
+    both the short-ring path and the counted tail), both 16-bit types.  Tiled and row-major weights must agree bit
+    for bit where both run the streaming kernel (K >= 512), and both must match the oracle."""
+    import random
+
+    ops = _ops()
+    rnd = random.Random(seed)
+    for case in range(20):
+        E = rnd.choice([1, 2, 4, 8, 16, 33, 64])
+        k = min(rnd.choice([1, 2, 4, 6, 8]), E)
+        T = rnd.choice([1, 2, 5, 8, 16, 33, 64, 100, 257])
+        H = 128 * rnd.choice([1, 2, 3, 4, 8, 11, 16])
+        I = 128 * rnd.choice([1, 2, 3, 4, 5, 11])
+        dtype = rnd.choice([torch.bfloat16, torch.float16])
+        g = torch.Generator().manual_seed(seed * 100003 + case * 7919 + E)
+        noise = torch.rand(T, E, generator=g) + torch.arange(E).float().pow(1.3) * rnd.choice([0.0, 0.03, 0.2])
+        se, ss, off = oracle.sort_bin(noise.argsort(dim=1)[:, :k], E)
+        x = _rand((T, H), 1.0, dtype, g)
+        w_fc_q, fc_scale = oracle.quantize_fp8_per_channel(torch.randn(E, 2 * I, H, generator=g) * 0.02)
+        w_pj_q, pj_scale = oracle.quantize_fp8_per_channel(torch.randn(E, H, I, generator=g) * 0.02)
+        xd, ssd, offd = x.to(device), ss.to(device), off.to(device)
+        fc_d, fcs_d, pj_d, pjs_d = (t.to(device) for t in (w_fc_q, fc_scale, w_pj_q, pj_scale))
+        print(f"fp8 random seed {seed} case {case}: T={T} E={E} k={k} H={H} I={I} {dtype}", flush=True)
+        act_t = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd)
+        act_r = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd)
+        o_t = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd)
+        o_r = ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd)
+        if H >= 512:
+            assert torch.equal(act_t, act_r), (case, "up")
+        if I >= 512:
+            assert torch.equal(o_t, o_r), (case, "down")
+        ref_act = oracle.swiglu(oracle.scattered_experts_oracle(x, oracle.dequant_fp8(w_fc_q, fc_scale), k, se, ss, off,
+                                                                grouped_out=True))
+        ref_o = oracle.scattered_experts_oracle(act_t.cpu(), oracle.dequant_fp8(w_pj_q, pj_scale), 1, se, ss, off,
+                                                grouped_in=True)
+        for name, got, ref in (("up", act_t, ref_act), ("up row-major", act_r, ref_act), ("down", o_t, ref_o),
+                               ("down row-major", o_r, ref_o)):
+            err = (got.cpu().float() - ref).abs().max().item()
+            assert err <= 2e-2 * ref.abs().max().item() + 2e-3, (case, name, err)
