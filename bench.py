@@ -16,7 +16,17 @@ Zipf(1.1) expert load).  One JSON line is printed:
                     branch) in fp32 on the host cores, on a bounded token sample of the same workload
 * ``workloads``     (default run only) the other four parity configurations, measured the same way in a few
                     seconds each: ms per step, the dominant kernel's roofline fraction, both grouped GEMMs
-                    together, and the whole layer's algorithmic bytes over HBM peak (the decode target)
+                    together, and the whole layer's algorithmic bytes over HBM peak (the decode target); the
+                    decode workload also with the latency of ONE forward (launch, synchronise; median) and of
+                    one replay of the forward captured in a HIP graph
+* ``ceilings``      (default run only) what this GPU does, in this process, on work of the same size with no
+                    gather, no expert boundaries and no activation: the vendor library's dense bf16 GEMM
+                    (torch.mm) of both grouped GEMMs' shapes on the same random data, and a 1 GiB copy
+* ``training``      (default run, or --backward) one training step of the layer (forward + backward for x and
+                    every parameter) through the kernel branch and through the eager branch, with the stage
+                    times of the kernel branch and the weight-gradient kernel's rate
+* ``block_fusion``  (default run only) the two fusions with the transformer block around the layer, each against
+                    the separate calls: RMSNorm + router, and combine + shared-expert sum + residual tail
 """
 
 import argparse
@@ -174,6 +184,7 @@ def measure_compact(name, device, steps=20, warmup=5):
         up_bytes = touched * (2 * w.I * w.H) + touched * 2 * w.I * 4 + w.T * w.H * 2 + L * w.I * 2 + L * 4 + w.E * 4
         out["kernel"], out["bound"] = "up_swiglu_fp8", "hbm"
         out["frac"] = up_bytes / (stages["up_swiglu_fp8"] * 1e-3) / 1e9 / PEAK_HBM_GBS
+        out.update(measure_latency(m, x))
     else:
         peak = PEAK_FP32_TFLOPS if w.dtype == torch.float32 else PEAK_BF16_TFLOPS
         out["kernel"], out["bound"] = "up_swiglu", "mfma"
@@ -182,6 +193,210 @@ def measure_compact(name, device, steps=20, warmup=5):
                                   / 1e12 / peak)
     del m, x, inputs
     torch.cuda.empty_cache()
+    return out
+
+
+def _time_ms(fn, iters, warmup=3):
+    """Average duration of ``fn()`` over ``iters`` launches between two HIP events on the current stream."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
+def measure_ceilings(w, inputs, device, iters=20):
+    """What the same GPU does in the same process on the same amount of work without the layer's structure:
+    the vendor library's dense GEMM (torch.mm, bf16) for both grouped GEMMs' shapes -- L rows of N(0,1) data against
+    ONE expert's N(0,0.02) weights, no gather, no expert boundaries, no SwiGLU, contiguous output -- and a 1 GiB
+    device-to-device copy.  The grouped kernels cannot be expected to beat these; the distance to them is what the
+    gather, the expert tails and the epilogue cost."""
+    import torch
+
+    L = w.T * w.k
+    g = torch.Generator(device="cpu").manual_seed(99)
+    out = {}
+    w_fc = inputs["w_fc"][0].to(device)          # (2I, H)
+    w_proj = inputs["w_proj"][0].to(device)      # (H, I)
+    xs = torch.randn(1024, w.H, generator=g).to(w.dtype).to(device).repeat(L // 1024 + 1, 1)[:L].contiguous()
+    # (rows repeat every 1024: the data stays random for the multipliers, and drawing 400 M normals on the host
+    #  would take longer than everything else in this file)
+    xs += torch.arange(L, device=device, dtype=torch.float32).mul_(1e-6).to(w.dtype).unsqueeze(1)
+    acts = torch.randn(1024, w.I, generator=g).mul_(0.3).to(w.dtype).to(device).repeat(L // 1024 + 1, 1)[:L].contiguous()
+    up_out = torch.empty((L, 2 * w.I), dtype=w.dtype, device=device)
+    down_out = torch.empty((L, w.H), dtype=w.dtype, device=device)
+    peak = PEAK_BF16_TFLOPS
+    ms = _time_ms(lambda: torch.mm(xs, w_fc.t(), out=up_out), iters)
+    fl = 2.0 * L * w.H * 2 * w.I
+    out["dense_up_gemm"] = {"shape": f"({L} x {w.H}) @ ({2 * w.I} x {w.H})^T", "ms": ms,
+                            "tflops": fl / (ms * 1e-3) / 1e12, "frac": fl / (ms * 1e-3) / 1e12 / peak}
+    ms2 = _time_ms(lambda: torch.mm(acts, w_proj.t(), out=down_out), iters)
+    fl2 = 2.0 * L * w.I * w.H
+    out["dense_down_gemm"] = {"shape": f"({L} x {w.I}) @ ({w.H} x {w.I})^T", "ms": ms2,
+                              "tflops": fl2 / (ms2 * 1e-3) / 1e12, "frac": fl2 / (ms2 * 1e-3) / 1e12 / peak}
+    out["dense_both_gemms_frac"] = (fl + fl2) / ((ms + ms2) * 1e-3) / 1e12 / peak
+    del xs, acts, up_out, down_out
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=device).random_(0, 255)
+    dst = torch.empty_like(src)
+    ms3 = _time_ms(lambda: dst.copy_(src), 10)
+    out["copy_1gib"] = {"ms": ms3, "gbs_read_plus_write": 2.0 * (1 << 30) / (ms3 * 1e-3) / 1e9,
+                        "frac": 2.0 * (1 << 30) / (ms3 * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    out["note"] = ("torch.mm (vendor dense bf16 GEMM) and Tensor.copy_ timed with HIP events in this process; "
+                   "frac is of the 2.5 PFLOP/s bf16 MFMA peak / the 8 TB/s HBM peak")
+    del src, dst
+    torch.cuda.empty_cache()
+    return out
+
+
+def measure_training(m, x, w, steps, full=False):
+    """One training step of the layer (forward + backward for the input and every parameter, a synthetic upstream
+    gradient, the auxiliary loss included) through the kernel branch and through the eager branch."""
+    import torch
+
+    from dolomite_engine_amd import Kernel, enable_kernels, ops
+    from dolomite_engine_amd.loss import clear_aux_loss, get_aux_loss
+
+    m.train()
+    xg = x.clone().requires_grad_(True)
+    dy = torch.randn_like(x)
+
+    def train_step(kernels: bool):
+        m.zero_grad(set_to_none=True)
+        xg.grad = None
+        clear_aux_loss()
+        if kernels:
+            with enable_kernels([Kernel.scattermoe]):
+                out_ = m(xg)
+        else:
+            out_ = m(xg)
+        ((out_ * dy).sum() + 0.01 * get_aux_loss()).backward()
+
+    train = {}
+    # kernels: the up-projection's pre-activation is kept for the backward (the module's default);
+    # kernels_recompute: it is recomputed there (MoE.keep_preactivation = False)
+    variants = [("kernels", True), ("eager", False)]
+    if full:
+        variants.insert(1, ("kernels_recompute", True))
+    for name, kernels in variants:
+        m.keep_preactivation = name != "kernels_recompute"
+        torch.cuda.reset_peak_memory_stats()
+        for _ in range(3):
+            train_step(kernels)
+        torch.cuda.synchronize()
+        train["peak_mem_gib_" + name] = torch.cuda.max_memory_allocated() / 2 ** 30
+        n = max(3, steps // 5)
+        t0 = time.perf_counter()
+        for _ in range(n):
+            train_step(kernels)
+        torch.cuda.synchronize()
+        train["ms_per_step_fwd_bwd_" + name] = (time.perf_counter() - t0) / n * 1e3
+    m.keep_preactivation = True
+    timer = StageTimer()
+    ops.set_stage_timer(timer)
+    for _ in range(5):
+        train_step(True)
+    stages = timer.per_step(5)
+    ops.set_stage_timer(None)
+    train["stages_ms_fwd_bwd"] = stages
+    train["kernel_stages_ms_sum"] = sum(stages.values())
+    if "grouped_wgrad" in stages:
+        # both weight gradients: d_w_fc 2 * L * 2I * H flops, d_w_proj 2 * L * H * I
+        fl = 6.0 * w.T * w.k * w.H * w.I
+        train["wgrad_tflops"] = fl / (stages["grouped_wgrad"] * 1e-3) / 1e12
+        train["wgrad_frac"] = train["wgrad_tflops"] / PEAK_BF16_TFLOPS
+    m.eval()
+    m.zero_grad(set_to_none=True)
+    del xg, dy
+    torch.cuda.empty_cache()
+    return train
+
+
+def measure_block_fusion(m, x, w, iters=30):
+    """The two fusions with the transformer block around the layer (ln_2 in front, shared-expert sum / m_residual /
+    residual add behind), each against the separate calls it replaces."""
+    import torch
+    import torch.nn.functional as F
+
+    from dolomite_engine_amd import ops
+
+    out = {}
+    with torch.no_grad():
+        gamma = torch.ones(w.H, dtype=w.dtype, device=x.device)
+        bias = m.router_logit_bias
+        if ops.rmsnorm_router_fused_supported(x, w.E, w.k):
+            def unfused():
+                xn = F.rms_norm(x, (w.H,), gamma, 1e-5)
+                return ops.router_fused(xn, m.gate.weight, w.k, bias=bias)
+
+            out["rmsnorm_plus_router_ms"] = _time_ms(unfused, iters)
+            out["rmsnorm_router_fused_ms"] = _time_ms(
+                lambda: ops.rmsnorm_router_fused(x, gamma, 1e-5, m.gate.weight, w.k, bias=bias), iters)
+        L = w.T * w.k
+        o = torch.randn(1024, w.H, device=x.device).to(w.dtype).repeat(L // 1024, 1)
+        gates = torch.rand(w.T, w.k, device=x.device).to(w.dtype)
+        shared = torch.randn_like(x)
+        residual = torch.randn_like(x)
+        out["combine_ms"] = _time_ms(lambda: ops.combine(o, gates), iters)
+        out["combine_then_shared_scale_residual_ms"] = _time_ms(
+            lambda: (ops.combine(o, gates) + shared) * 0.22 + residual, iters)
+        out["combine_block_tail_fused_ms"] = _time_ms(lambda: ops.combine(o, gates, shared, residual, 0.22), iters)
+        del o, gates, shared, residual
+    torch.cuda.empty_cache()
+    return out
+
+
+def measure_latency(m, x, reps=300):
+    """One forward at a time: launch, wait for the device, repeat; the median.  And the same forward captured into
+    a HIP graph, one replay at a time."""
+    import torch
+
+    from dolomite_engine_amd import Kernel, enable_kernels
+
+    out = {}
+    with torch.no_grad(), enable_kernels([Kernel.scattermoe]):
+        for _ in range(20):
+            y = m(x)
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            y = m(x)
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+        out["latency_ms"] = sorted(ts)[len(ts) // 2] * 1e3
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            m(x)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_static = m(x)
+        for _ in range(20):
+            graph.replay()
+        torch.cuda.synchronize()
+        if not torch.equal(y_static, y):
+            raise RuntimeError("graph replay differs from the eager forward")
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+        out["graph_replay_latency_ms"] = sorted(ts)[len(ts) // 2] * 1e3
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            graph.replay()
+        torch.cuda.synchronize()
+        out["graph_replay_ms"] = (time.perf_counter() - t0) / reps * 1e3
+        del graph, y_static
     return out
 
 
@@ -331,51 +546,9 @@ def main():
         idx = m._compute_routing_weights(x)[2]
         counts = torch.bincount(idx.flatten().long(), minlength=E).cpu()
 
-    train = None
-    if args.backward:
-        if w.fp8:
-            print("bench.py: --backward needs a 16-bit workload", file=sys.stderr)
-            sys.exit(2)
-        from dolomite_engine_amd.loss import clear_aux_loss, get_aux_loss
-
-        m.train()
-        xg = x.clone().requires_grad_(True)
-        dy = torch.randn_like(x)
-
-        def train_step(kernels: bool):
-            m.zero_grad(set_to_none=True)
-            xg.grad = None
-            clear_aux_loss()
-            if kernels:
-                with enable_kernels([Kernel.scattermoe]):
-                    out_ = m(xg)
-            else:
-                out_ = m(xg)
-            ((out_ * dy).sum() + 0.01 * get_aux_loss()).backward()
-
-        train = {}
-        # kernels: the up-projection's pre-activation is kept for the backward (the module's default);
-        # kernels_recompute: it is recomputed there (MoE.keep_preactivation = False)
-        for name, kernels in (("kernels", True), ("kernels_recompute", True), ("eager", False)):
-            m.keep_preactivation = name != "kernels_recompute"
-            torch.cuda.reset_peak_memory_stats()
-            for _ in range(3):
-                train_step(kernels)
-            torch.cuda.synchronize()
-            train["peak_mem_gib_" + name] = torch.cuda.max_memory_allocated() / 2 ** 30
-            n = max(3, args.steps // 5)
-            t0 = time.perf_counter()
-            for _ in range(n):
-                train_step(kernels)
-            torch.cuda.synchronize()
-            train["ms_per_step_fwd_bwd_" + name] = (time.perf_counter() - t0) / n * 1e3
-        timer = StageTimer()
-        ops.set_stage_timer(timer)
-        for _ in range(5):
-            train_step(True)
-        train["stages_ms_fwd_bwd"] = timer.per_step(5)
-        ops.set_stage_timer(None)
-        m.eval()
+    if (args.backward or (w.name == "granite-3b-a800m" and not args.no_other_workloads)) and w.fp8:
+        print("bench.py: --backward needs a 16-bit workload", file=sys.stderr)
+        sys.exit(2)
 
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = T / (elapsed / args.steps)
@@ -419,14 +592,20 @@ def main():
         "stages_ms": stages,
         "roofline": roofline,
     }
-    if w.name == "granite-3b-a800m" and not args.no_other_workloads:
+    default_extras = w.name == "granite-3b-a800m" and not args.no_other_workloads
+    if w.fp8:
+        out.update(measure_latency(m, x))
+    if default_extras:
+        out["ceilings"] = measure_ceilings(w, inputs, device)
+        out["block_fusion"] = measure_block_fusion(m, x, w)
+    if args.backward or default_extras:
+        out["training"] = measure_training(m, x, w, args.steps, full=args.backward)
+    if default_extras:
         del m, x
         torch.cuda.empty_cache()
         out["workloads"] = {n: measure_compact(n, device) for n in oracle.WORKLOADS if n != w.name}
     if graph_ms is not None:
         out["ms_per_step_graph_replay"] = graph_ms
-    if train is not None:
-        out["training"] = train
     if not args.no_cpu_baseline:
         sample = args.cpu_sample_tokens or min(T, 8192)
         out["cpu_baseline"] = cpu_baseline(w, inputs, sample)

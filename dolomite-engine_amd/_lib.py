@@ -44,6 +44,7 @@ SIGNATURES: dict[str, tuple] = {
     "mi_moe_up_swiglu": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "mi_moe_up_swiglu_cfg": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mi_moe_grouped_gemm_workspace_bytes": (_sz, []),
+    "mi_moe_grouped_gemm_splits": (_i, [_i, _i]),
     "mi_moe_scattered_gemm_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "mi_moe_scattered_gemm_wt_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "mi_moe_up_swiglu_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),

@@ -706,6 +706,13 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GemmArgs 
 #define PERSIST_SPLIT_MIN_SLICES 32
 #define PERSIST_WS_TILE_BYTES (256 * 256 * 4)
 
+// whether a contraction of length K can be shortened by PERSIST_SPLIT_MIN_SAVED slices at all (launch_persistent
+// applies the same rule, plus one on the grid)
+static bool persistent_may_split(int K) {
+  const int nk = K / 32;
+  return nk - nk / PERSIST_SPLIT_MAX >= PERSIST_SPLIT_MIN_SAVED;
+}
+
 // Which tiles a workgroup runs.  Workgroup b sits on XCD b % 8 (the hardware deals workgroup ids round-robin to the
 // XCDs) in slot b / 8.  Two ways of dealing the band-ordered tile list to them:
 //   * contiguous (the default): XCD x owns the x-th eighth of the list and deals it to its slots in turn, so the
@@ -1410,10 +1417,7 @@ static int launch_persistent(GemmArgs a, hipStream_t s) {
   long grid = cus < max_tiles ? cus : max_tiles;
   grid = (grid + 7) / 8 * 8;
   // no contraction length that a split could shorten by PERSIST_SPLIT_MIN_SAVED slices, or one slot per XCD
-  {
-    const int nk = a.K / 32;
-    if (nk - nk / PERSIST_SPLIT_MAX < PERSIST_SPLIT_MIN_SAVED || grid < 16) a.ws = nullptr;
-  }
+  if (!persistent_may_split(a.K) || grid < 16) a.ws = nullptr;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, a);
   if ((rc = mi_launch_status()) != MI_MOE_OK || a.ws == nullptr) return rc;
   // the tiles that were cut: at most half of the slots of a round that was split hold tiles (rounded up: an odd
@@ -1429,6 +1433,10 @@ extern "C" size_t mi_moe_grouped_gemm_workspace_bytes(void) {
   int cus = 0;
   if (mi_cu_count(&cus) != MI_MOE_OK) return 0;
   return (size_t)((cus + 7) / 8 * 8) * PERSIST_WS_TILE_BYTES;
+}
+
+extern "C" int mi_moe_grouped_gemm_splits(int K, int dtype) {
+  return (dtype == MI_MOE_BF16 || dtype == MI_MOE_F16) && K > 0 && K % 32 == 0 && persistent_may_split(K);
 }
 
 static int check_ws(const void* ws, size_t ws_bytes) {

@@ -25,8 +25,8 @@ _TIMER = None
 _WARNED: set = set()
 
 
-def _warn_once(key: str, message: str) -> None:
-    """Slow paths are taken loudly: one warning per process and kind."""
+def _warn_once(key, message: str) -> None:
+    """Slow paths are taken loudly: one warning per process and key (reason, shape, dtype)."""
     if key not in _WARNED:
         _WARNED.add(key)
         import warnings
@@ -276,22 +276,29 @@ def sort_bin(selected_experts: torch.Tensor, num_experts: int):
 
 
 _GEMM_WS: dict = {}
+_GEMM_WS_MAX = 16
 
 
-def _gemm_workspace(device: torch.device, enabled: bool = True):
+def _gemm_workspace(device: torch.device, K: int, dtype: torch.dtype, enabled: bool = True):
     """(tensor, bytes) of the workspace that lets the persistent grouped GEMM cut the tiles of its last, partly
-    filled round along K (mi_moe_grouped_gemm_workspace_bytes: one fp32 partial tile per CU, 64 MiB on 256 CUs).
-    One per device and stream, kept for the life of the process; its contents carry nothing between calls."""
-    if not enabled:
+    filled round along K (mi_moe_grouped_gemm_workspace_bytes: one fp32 partial tile per CU, 64 MiB on 256 CUs), or
+    (None, 0) when the library would not use it for this contraction length and dtype (mi_moe_grouped_gemm_splits:
+    16-bit and K >= 5120) -- most layers never allocate one.
+
+    One buffer per (device, stream), created on first use and NEVER released: a HIP graph captured on that stream
+    holds the buffer's address for as long as it can be replayed.  After _GEMM_WS_MAX buffers further streams get
+    none (their calls run every tile whole, which is only slower)."""
+    if not enabled or dtype not in (torch.float16, torch.bfloat16):
+        return None, 0
+    lib = _lib.load()
+    if not lib.mi_moe_grouped_gemm_splits(K, _code(dtype)):
         return None, 0
     key = (device.index, _stream())
     ws = _GEMM_WS.get(key)
     if ws is None:
-        n = _lib.load().mi_moe_grouped_gemm_workspace_bytes()
-        if n == 0:
+        n = lib.mi_moe_grouped_gemm_workspace_bytes()
+        if n == 0 or len(_GEMM_WS) >= _GEMM_WS_MAX:
             return None, 0
-        if len(_GEMM_WS) >= 16:  # streams come and go (graph captures): do not keep a buffer for each for ever
-            _GEMM_WS.clear()
         ws = torch.empty(n, dtype=torch.uint8, device=device)
         _GEMM_WS[key] = ws
     return ws, ws.numel()
@@ -325,7 +332,7 @@ def scattered_gemm(inputs: torch.Tensor, weight: torch.Tensor, k: int, sorted_sc
         raise ValueError("scattered inputs must have L / k rows")
     out = torch.empty((L, N), dtype=inputs.dtype, device=inputs.device)
     lib = _lib.load()
-    ws, ws_bytes = _gemm_workspace(inputs.device, split_k)
+    ws, ws_bytes = _gemm_workspace(inputs.device, K, inputs.dtype, split_k)
     if weight_kn:
         with _stage("scattered_gemm"):
             rc = lib.mi_moe_scattered_gemm_wt_ws(_ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N,
@@ -335,27 +342,40 @@ def scattered_gemm(inputs: torch.Tensor, weight: torch.Tensor, k: int, sorted_sc
             return out
         if rc not in (_lib.MI_MOE_EUNSUPPORTED, _lib.MI_MOE_EDTYPE, _lib.MI_MOE_EALIGN):
             check(rc)
-        _warn_once("weight_kn", f"scattered_gemm(weight_kn=True): the transposed-weight kernel does not take "
-                   f"K={K}, N={N}, E={E}, {inputs.dtype} ({lib.mi_moe_strerror(rc).decode()}); making a transposed "
-                   "copy of the weights for this call")
+        if inputs.dtype != torch.float32:
+            # (fp32 has no transposed-weight kernel: its transposed copy is the regular path, not a refusal)
+            _warn_once(("weight_kn", rc, K, N, inputs.dtype),
+                       f"scattered_gemm(weight_kn=True): the transposed-weight kernel does not take "
+                       f"K={K}, N={N}, E={E}, {inputs.dtype} ({lib.mi_moe_strerror(rc).decode()}); making a "
+                       "transposed copy of the weights for this call")
         weight = weight.transpose(1, 2).contiguous()
     with _stage("scattered_gemm"):
         rc = _gemm_or_slow(lambda c: lib.mi_moe_scattered_gemm_ws(
             _ptr(inputs), _ptr(weight), _ptr(out), _ptr(ss), _ptr(off), L, K, N, E, k, int(grouped_in),
-            int(grouped_out), _code(inputs.dtype), c, _ptr(ws), ws_bytes, _stream()), cfg, K, N, inputs.dtype)
+            int(grouped_out), _code(inputs.dtype), c, _ptr(ws), ws_bytes, _stream()), cfg, K, N, inputs.dtype,
+            inputs.shape[0])
         check(rc)
     return out
 
 
-def _gemm_or_slow(call, cfg: int, K: int, N: int, dtype: torch.dtype) -> int:
-    """Run ``call(cfg)``.  The library refuses 16-bit problems its matrix-core kernels cannot take instead of
-    silently running them on the one-thread-per-output kernel; the reference's op takes any shape, so for an
-    automatic pick (cfg < 0) that refusal is answered here by asking for that kernel explicitly -- with a warning."""
+def _gemm_or_slow(call, cfg: int, K: int, N: int, dtype: torch.dtype, rows: int) -> int:
+    """Run ``call(cfg)``.  The library refuses problems its matrix-core kernels cannot take instead of silently
+    running them on the one-thread-per-output kernel; the reference's op takes any shape, so for an automatic pick
+    (cfg < 0) a refusal for the shape's granularity (K not a multiple of a 16-byte chunk, N % 4) or for a misaligned
+    pointer is answered here by asking for that kernel explicitly -- with a warning per (reason, K, N, dtype) whose
+    text is the library's.  A well-formed problem that is refused only because an operand is too large for the
+    kernels' 32-bit element offsets is NOT sent there (it would run orders of magnitude slower without a word): it
+    raises, and the caller splits the rows."""
     rc = call(cfg)
     if cfg < 0 and rc in (_lib.MI_MOE_EUNSUPPORTED, _lib.MI_MOE_EALIGN):
-        _warn_once("slow_gemm", f"grouped GEMM with K={K}, N={N}, {dtype}: "
-                   f"{_lib.load().mi_moe_strerror(rc).decode()}; running the slow one-thread-per-output kernel "
-                   "(needs K % 8 == 0, N % 4 == 0 and 16-byte aligned tensors for the matrix-core kernels)")
+        chunk = 4 if dtype == torch.float32 else 8
+        if rc == _lib.MI_MOE_EUNSUPPORTED and K % chunk == 0 and N % 4 == 0:
+            raise _lib.MiMoeError(
+                f"grouped GEMM with {rows} input rows, K={K}, N={N}, {dtype}: an operand has 2^31 or more elements, "
+                "beyond the 32-bit element offsets of the matrix-core kernels; split the call by rows")
+        _warn_once(("slow_gemm", rc, K, N, dtype),
+                   f"grouped GEMM with K={K}, N={N}, {dtype}: {_lib.load().mi_moe_strerror(rc).decode()}; running "
+                   "the one-thread-per-output kernel instead")
         rc = call(3)
     return rc
 
@@ -608,11 +628,11 @@ def up_swiglu(x: torch.Tensor, w_fc: torch.Tensor, k: int, sorted_scattered_idxs
         raise ValueError("x must have L / k rows")
     act = torch.empty((L, I2 // 2), dtype=x.dtype, device=x.device)
     lib = _lib.load()
-    ws, ws_bytes = _gemm_workspace(x.device, split_k)
+    ws, ws_bytes = _gemm_workspace(x.device, H, x.dtype, split_k)
     with _stage("up_swiglu"):
         check(_gemm_or_slow(lambda c: lib.mi_moe_up_swiglu_ws(
             _ptr(x), _ptr(w_fc), _ptr(act), _ptr(ss), _ptr(off), L, H, I2 // 2, E, k, _code(x.dtype), c, _ptr(ws),
-            ws_bytes, _stream()), cfg, H, I2 // 2, x.dtype))
+            ws_bytes, _stream()), cfg, H, I2 // 2, x.dtype, x.shape[0]))
     return act
 
 

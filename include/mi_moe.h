@@ -204,8 +204,11 @@ int mi_moe_scattered_gemm_cfg(const void* in, const void* w, void* out, const in
  * without a workspace.  ws: mi_moe_grouped_gemm_workspace_bytes() bytes (one partial tile per CU of the current
  * device; 0 if there is no device), 16-byte aligned, MI_MOE_EWORKSPACE / MI_MOE_EALIGN otherwise; contents need
  * no initialisation and carry nothing between calls; calls that overlap in time need separate workspaces.
+ * mi_moe_grouped_gemm_splits(K, dtype) tells a caller whether a product of contraction length K and that element
+ * type can use the workspace at all (1) or would ignore it (0), so that it need not allocate one.
  */
 size_t mi_moe_grouped_gemm_workspace_bytes(void);
+int mi_moe_grouped_gemm_splits(int K, int dtype);
 int mi_moe_scattered_gemm_ws(const void* in, const void* w, void* out, const int32_t* sorted_scattered,
                              const int32_t* expert_offsets, int L, int K, int N, int E, int k, int grouped_in,
                              int grouped_out, int dtype, int cfg, void* ws, size_t ws_bytes, mi_moe_stream_t stream);

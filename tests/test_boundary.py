@@ -174,6 +174,41 @@ def test_enable_kernels_replaces_and_restores():
     assert not is_kernel_allowed(Kernel.scattermoe)  # restored even when the block raises
 
 
+def test_enable_all_cute_kernels_environment_switch(monkeypatch):
+    """lm_engine/kernels.py:14-19, 75-76: ENABLE_ALL_CUTE_KERNELS, read when the module is imported, switches every
+    kernel on for the whole process -- but only where the kernels can run."""
+    from dolomite_engine_amd import kernels
+
+    everything = {k for k in Kernel if k != Kernel.ladder_residual_overlapped_layer}
+    before = kernels._KERNELS
+    started_with = os.environ.get("ENABLE_ALL_CUTE_KERNELS", "0").lower() in ("1", "true")
+    really_available = kernels._kernels_available()
+    try:
+        for value, available, expect in [(None, True, False), ("0", True, False), ("false", True, False),
+                                         ("1", False, False), ("1", True, True), ("TRUE", True, True)]:
+            kernels._KERNELS = set()
+            if value is None:
+                monkeypatch.delenv("ENABLE_ALL_CUTE_KERNELS", raising=False)
+            else:
+                monkeypatch.setenv("ENABLE_ALL_CUTE_KERNELS", value)
+            monkeypatch.setattr(kernels, "_kernels_available", lambda available=available: available)
+            assert kernels._enable_all_from_environment() is expect
+            assert kernels._KERNELS == (everything if expect else set())
+            assert is_kernel_allowed(Kernel.scattermoe) is expect
+            assert not is_kernel_allowed(Kernel.ladder_residual_overlapped_layer)
+            if expect:  # a context still replaces the set and puts "everything" back
+                with enable_kernels([Kernel.rmsnorm_cute]):
+                    assert not is_kernel_allowed(Kernel.scattermoe)
+                assert is_kernel_allowed(Kernel.scattermoe)
+        monkeypatch.setenv("ENABLE_ALL_CUTE_KERNELS", "maybe")
+        with pytest.raises(ValueError):
+            kernels._enable_all_from_environment()
+    finally:
+        kernels._KERNELS = before
+    # this process was started without the variable (or without a GPU): nothing is on by default
+    assert kernels._ENABLE_ALL_KERNELS is (started_with and really_available)
+
+
 # ---------------------------------------------------------------------------------------------------
 # module interface
 # ---------------------------------------------------------------------------------------------------

@@ -251,6 +251,60 @@ def test_split_k_of_the_last_round(device, form, name, counts, K, N):
     assert bool(one_step.all())
 
 
+def test_split_k_workspace_outlives_a_captured_graph(device):
+    """A product long enough to be cut along K (K >= 5120) is captured into a HIP graph, which bakes the address of
+    the workspace into the graph.  Calls on more than sixteen further streams must neither release that buffer nor
+    hand it to someone else: every later replay still equals the eager result, also after the caching allocator
+    has been churned.  Shorter contractions never get a workspace."""
+    ops = _ops()
+    counts, K, N = [5000, 5000, 5000, 5000], 8192, 1024
+    g = torch.Generator().manual_seed(77)
+    E, L = len(counts), sum(counts)
+    off = torch.tensor(counts).cumsum(0).to(torch.int32).to(device)
+    ss = torch.randperm(L, generator=g).to(torch.int32).to(device)
+    inp = (torch.randn(L, K, generator=g) * 0.5).to(torch.bfloat16).to(device)
+    w = (torch.randn(E, N, K, generator=g) * 0.05).to(torch.bfloat16).to(device)
+    print("split-K workspace under graph capture", flush=True)
+    assert ops._gemm_workspace(torch.device(device), 512, torch.bfloat16)[0] is None
+    assert ops._gemm_workspace(torch.device(device), 8192, torch.float32)[0] is None
+    eager = ops.scattered_gemm(inp, w, 1, ss, off, True, False, cfg=7)
+    torch.cuda.synchronize()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.scattered_gemm(inp, w, 1, ss, off, True, False, cfg=7)   # creates the side stream's workspace
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = ops.scattered_gemm(inp, w, 1, ss, off, True, False, cfg=7)
+    held = {k: v.data_ptr() for k, v in ops._GEMM_WS.items()}
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, eager)
+
+    small_in = inp[:, :5120].contiguous()
+    small_w = w[:, :256, :5120].contiguous()
+    for i in range(20):   # more streams than the cache keeps buffers for
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            ops.scattered_gemm(small_in, small_w, 1, ss, off, True, False, cfg=7)
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+        junk = torch.full((96 << 20,), 0x7f, dtype=torch.uint8, device=device)  # would land on a released workspace
+        del junk
+        if i % 5 == 4:
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), f"replay after {i + 1} further streams"
+    for k, ptr in held.items():   # nothing that existed at capture time was dropped or replaced
+        assert ops._GEMM_WS[k].data_ptr() == ptr
+    assert len(ops._GEMM_WS) <= ops._GEMM_WS_MAX
+
+
 @pytest.mark.parametrize("seed", [1, 2, 3, 4])
 def test_persistent_kernel_random_shapes(device, seed):
     """The persistent kernel's scheduling (tile order by XCD in both forms, last round cut along K, finishing

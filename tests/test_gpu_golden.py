@@ -1,8 +1,12 @@
-"""The HIP path on committed golden data -- evidence that does not pass through oracle/ at run time.
+"""The HIP path on committed golden data.
 
-* tests/golden/workloads.json (written by tests/golden/make_workload_goldens.py): the five benchmark / parity
-  workloads at full size; the device's routing must reproduce the recorded histogram and first-token routing
-  exactly and the layer output the recorded slice and checksums of the fp32 result.
+* tests/golden/workloads.json (written by tests/golden/make_workload_goldens.py FROM THE ORACLE, on inputs that
+  oracle.make_inputs draws again here): the five benchmark / parity workloads at full size; the device's routing
+  must reproduce the recorded histogram and first-token routing exactly and the layer output the recorded slice and
+  checksums of the fp32 result.  This is the oracle's answer frozen -- it guards against drift of the oracle, the
+  generator or the kernels between machines and versions; it is not evidence independent of the oracle.
+* The two .npz files below ARE independent of oracle/: neither their inputs nor their expected outputs pass
+  through it.
 * tests/golden/granitemoe_h32_e8_k{2,8}.npz (written by tests/golden/make_golden.py from transformers'
   GraniteMoeMoE, which the reference asserts its eager branch equals:
   tests/hf_models/single_gpu/model_conversion_test.py:60-103): loaded into the module directly and through a

@@ -32,7 +32,7 @@ def test_generated_inputs_match_recorded_hashes(name):
     assert got == rec["sha256"], "the CPU generator no longer produces the recorded tensors"
 
 
-@pytest.mark.parametrize("name", ["tiny-fp32", "granite-1b-a400m", "granite-3b-a800m", "decode-fp8"])
+@pytest.mark.parametrize("name", NAMES)
 def test_oracle_routing_matches_recorded_routing(name):
     rec = workload_goldens()[name]["routing"]
     w = oracle.WORKLOADS[name]
