@@ -30,6 +30,7 @@ SIGNATURES: dict[str, tuple] = {
     "mi_moe_router_topk_softmax": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "mi_moe_router_fused_workspace_bytes": (_sz, [_i, _i, _i]),
     "mi_moe_router_fused": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "mi_moe_router_dlogits": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "mi_moe_router_fused_sort_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mi_moe_router_fused_sort": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "mi_moe_rmsnorm_router_fused_supported": (_i, [_i, _i, _i, _i]),

@@ -24,7 +24,10 @@ from . import ops
 
 
 class ScatteredSwiGLUExperts(torch.autograd.Function):
-    """y[t] = sum_j gates[t, j] * ( swiglu(x[t] @ w_fc[e]^T) @ w_proj[e]^T ),  e = expert of slot (t, j)."""
+    """y[t] = sum_j gates[t, j] * ( swiglu(x[t] @ w_fc[e]^T) @ w_proj[e]^T ),  e = expert of slot (t, j).
+
+    ``gates=None`` (needs k == 1): no router weights and no combine pass, y is the rows of the down-projection in
+    flat-slot order -- the shared experts (moe.py:311-315) run this way as one expert that owns every token."""
 
     @staticmethod
     def forward(ctx, x, w_fc, w_proj, gates, sorted_scattered, expert_offsets, k, keep_preactivation=True):
@@ -35,7 +38,12 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
         else:
             act = ops.up_swiglu(x, w_fc, k, sorted_scattered, expert_offsets)
         o = ops.scattered_gemm(act, w_proj, 1, sorted_scattered, expert_offsets, True, False)
-        y = ops.combine(o, gates)
+        if gates is None:
+            if k != 1:
+                raise ValueError("gates=None needs k == 1")
+            y = o
+        else:
+            y = ops.combine(o, gates)
         ctx.save_for_backward(x, w_fc, w_proj, gates, sorted_scattered, expert_offsets, h)
         ctx.k = k
         return y
@@ -58,16 +66,20 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
         if h is None:
             h = ops.scattered_gemm(x, w_fc, k, ss, off, False, True)
         if half:
-            d_h, act_g, d_gates = ops.swiglu_backward(h, d_act, gates, ss, want_act=True, want_gate_grad=True)
+            d_h, act_g, d_gates = ops.swiglu_backward(h, d_act, gates, ss if gates is not None else None,
+                                                      want_act=True, want_gate_grad=gates is not None)
         else:
             ssl = ss.long()
-            g_sorted = gates.reshape(-1)[ssl].float().unsqueeze(-1)
             up, gate, da = h[:, :I].float(), h[:, I:].float(), d_act.float()
             sig = torch.sigmoid(gate)
             a = up * gate * sig
-            d_gates = torch.empty(T * k, dtype=torch.float32, device=x.device)
-            d_gates[ssl] = (da * a).sum(dim=1)
-            d_gates = d_gates.view(T, k).to(gates.dtype)
+            if gates is None:
+                g_sorted, d_gates = 1.0, None
+            else:
+                g_sorted = gates.reshape(-1)[ssl].float().unsqueeze(-1)
+                d_gates = torch.empty(T * k, dtype=torch.float32, device=x.device)
+                d_gates[ssl] = (da * a).sum(dim=1)
+                d_gates = d_gates.view(T, k).to(gates.dtype)
             da = da * g_sorted
             d_h = torch.cat([da * gate * sig, da * up * sig * (1.0 + gate * (1.0 - sig))], dim=1).to(x.dtype)
             act_g = (a * g_sorted).to(x.dtype)
@@ -76,7 +88,12 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
 
         # gradient w.r.t. x: every slot's contribution in flat-slot order, then the k slots of a token summed
         dx_slots = ops.scattered_gemm(d_h, w_fc, 1, ss, off, True, False, weight_kn=True)
-        dx = ops.combine(dx_slots, torch.ones_like(gates))
+        if k == 1:
+            dx = dx_slots
+        elif half:
+            dx = ops.combine(dx_slots, torch.ones((T, k), dtype=x.dtype, device=x.device))
+        else:
+            dx = dx_slots.view(T, k, H).sum(dim=1)
         del dx_slots
 
         # weight gradients: per expert X^T dY over that expert's rows
@@ -160,3 +177,38 @@ class SwitchAuxLoss(torch.autograd.Function):
     def backward(ctx, grad):
         logits, loss_w = ctx.saved_tensors
         return ops.aux_loss_backward(logits.detach(), loss_w, grad), None
+
+
+class FusedRouter(torch.autograd.Function):
+    """MoE._compute_routing_weights (moe.py:246-257) as one differentiable function on this package's kernels:
+
+        logits = x @ gate_w^T (+ bias) in x.dtype;  experts = top-k;  gates = softmax over the k picked logits
+
+    Returns (logits, gates, experts).  The backward takes the gradients that arrive at ``gates`` (from the expert
+    combine) and at ``logits`` (from the auxiliary loss), forms d logits in one element-wise kernel and runs the two
+    products d x = d logits @ gate_w and d gate_w = d logits^T @ x on the grouped GEMM / grouped weight-gradient
+    kernels as one expert that owns every token: no library GEMM in either direction."""
+
+    @staticmethod
+    def forward(ctx, x, gate_w, bias, k):
+        logits, gates, experts = ops.router_fused(x, gate_w, k, bias=bias, return_logits=True)
+        ctx.save_for_backward(x, gate_w, logits, experts)
+        ctx.mark_non_differentiable(experts)
+        return logits, gates, experts
+
+    @staticmethod
+    def backward(ctx, d_logits, d_gates, _):
+        x, gate_w, logits, experts = ctx.saved_tensors
+        T, H = x.shape
+        if d_logits is None and d_gates is None:
+            return None, None, None, None
+        dl = ops.router_dlogits(logits, experts, d_gates, d_logits)
+        rows = torch.arange(T, dtype=torch.int32, device=x.device)
+        off = torch.full((1,), T, dtype=torch.int32, device=x.device)
+        dx = dw = None
+        if ctx.needs_input_grad[0]:
+            # (T, E) @ (E, H): the gate weight transposed to (H, E) is the "(out, in)" weight of one expert
+            dx = ops.scattered_gemm(dl, gate_w.t().contiguous().unsqueeze(0), 1, rows, off, True, True)
+        if ctx.needs_input_grad[1]:
+            dw = ops.grouped_wgrad(dl, x, off)[0]
+        return dx, dw, None, None

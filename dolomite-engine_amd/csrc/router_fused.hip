@@ -721,16 +721,23 @@ extern "C" size_t mi_moe_router_fused_workspace_bytes(int T, int H, int E) {
   return (T < 0 || H < 1) ? 0 : router_ws_bytes(T, H);
 }
 
+// router_general.hip: fp32, 65 .. 256 experts, k up to 64
+int mi_router_general_ok(int H, int E, int k, int dtype);
+int mi_router_general(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k, int dtype,
+                      void* logits_out, void* gates, int32_t* idx, hipStream_t s);
+
 extern "C" int mi_moe_router_fused(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,
                                    int dtype, void* logits_out, void* gates_out, int32_t* idx_out, void* ws,
                                    size_t ws_bytes, mi_moe_stream_t stream) {
   if (T < 0 || H < 1 || E < 1 || k < 1 || k > E) return MI_MOE_ESHAPE;
-  if (E > 64 || k > ROUTER_KMAX || H % 16 != 0) return MI_MOE_EUNSUPPORTED;
-  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16 && dtype != MI_MOE_F32) return MI_MOE_EDTYPE;
+  const bool streaming = dtype != MI_MOE_F32 && E <= 64 && k <= ROUTER_KMAX && H % 16 == 0;
+  if (!streaming && !mi_router_general_ok(H, E, k, dtype)) return MI_MOE_EUNSUPPORTED;
   if (T == 0) return MI_MOE_OK;
   if (!x || !gate_w || !gates_out || !idx_out) return MI_MOE_ENULL;
   if (!mi_aligned(x, 16) || !mi_aligned(gate_w, 16)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (!streaming) return mi_router_general(x, gate_w, bias, T, H, E, k, dtype, logits_out, gates_out, idx_out, s);
   const size_t need = router_ws_bytes(T, H);
   if (ws != nullptr && need > 0) {  // few tokens and a workspace: K split across workgroups
     if (ws_bytes < need) return MI_MOE_EWORKSPACE;

@@ -7,41 +7,13 @@
 // the external continuous_count op used at moe.py:38-44.
 #include "common.h"
 #include "sort_block.h"
+#include "topk_row.h"
 
 // ------------------------------------------------------------------------------------------------
 // top-k softmax
 // ------------------------------------------------------------------------------------------------
 
-// Order-preserving map float -> uint32 (larger float <=> larger key); NaN is the largest key and
-// -0.0 is folded onto +0.0 so that it ties with it, as a floating-point comparison would.
-__device__ __forceinline__ uint32_t ordered_key(float v) {
-  uint32_t u = __float_as_uint(v);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;
-  if (u == 0x80000000u) u = 0u;
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-
-__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    uint32_t lo = __shfl_xor((uint32_t)v, off, MI_WAVE);
-    uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, MI_WAVE);
-    uint64_t o = ((uint64_t)hi << 32) | lo;
-    v = o > v ? o : v;
-  }
-  return v;
-}
-
-__device__ __forceinline__ float wave_sum_f32(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, MI_WAVE);
-  return v;
-}
-
-// One wavefront per row.  Lane l owns experts l, l+64, ... (VPL of them).  A candidate is the
-// 64-bit key (ordered(value) << 32) | ~expert, so a plain unsigned max implements "value
-// descending, expert index ascending".  Round j finds the j-th winner with a butterfly max; the
-// lane that owns it retires it.  Lane j keeps winner j, then lanes [0,k) do the softmax.
+// One wavefront per row; lane l owns experts l, l + 64, ... (topk_row.h).
 template <typename T, int VPL>
 __global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__ logits, int Trows, int E, int k,
                                                            T* __restrict__ gates, int32_t* __restrict__ idx) {
@@ -49,53 +21,13 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= Trows) return;
   const T* src = logits + (size_t)row * E;
-
   float vals[VPL];
-  uint64_t keys[VPL];
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    int e = lane + i * 64;
-    if (e < E) {
-      vals[i] = Elt<T>::load(src + e);
-      keys[i] = ((uint64_t)ordered_key(vals[i]) << 32) | (uint32_t)(~(uint32_t)e);
-    } else {
-      vals[i] = 0.f;
-      keys[i] = 0ull;  // below every real candidate (real keys have a non-zero low word)
-    }
+    const int e = lane + i * 64;
+    vals[i] = e < E ? Elt<T>::load(src + e) : 0.f;
   }
-
-  float my_val = 0.f;
-  int my_idx = 0;
-  for (int j = 0; j < k; ++j) {
-    uint64_t best = 0ull;
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) best = keys[i] > best ? keys[i] : best;
-    best = wave_max_u64(best);
-    int e = (int)(~(uint32_t)best);
-    // the owner retires the winner and publishes its value
-    float v = 0.f;
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-      if (keys[i] == best) {
-        v = vals[i];
-        keys[i] = 0ull;
-      }
-    }
-    v = __shfl(v, e & 63, MI_WAVE);
-    if (lane == j) {
-      my_val = v;
-      my_idx = e;
-    }
-  }
-
-  // softmax over the k winners in fp32; winner 0 is the maximum
-  float vmax = __shfl(my_val, 0, MI_WAVE);
-  float p = (lane < k) ? expf(my_val - vmax) : 0.f;
-  float denom = wave_sum_f32(p);
-  if (lane < k) {
-    Elt<T>::store(gates + (size_t)row * k + lane, p / denom);
-    idx[(size_t)row * k + lane] = my_idx;
-  }
+  topk_softmax_row<T, VPL>(vals, E, k, gates + (size_t)row * k, idx + (size_t)row * k);
 }
 
 template <typename T>

@@ -29,7 +29,7 @@ import torch.nn.functional as F
 
 from . import ops
 from .activations import GLUActivation, get_activation_function, is_glu
-from .autograd import ScatteredSwiGLUExperts, SwitchAuxLoss
+from .autograd import FusedRouter, ScatteredSwiGLUExperts, SwitchAuxLoss
 from .enums import Kernel
 from .kernels import is_kernel_allowed
 from .linear import ParameterizedLinear
@@ -314,6 +314,7 @@ class MoE(nn.Module):
         )
 
     def _use_fused_router(self, hidden_states: torch.Tensor) -> bool:
+        """The inference forms of the router kernel (sort or RMSNorm folded in, no logits kept)."""
         return (
             is_kernel_allowed(Kernel.scattermoe)
             and not self.training
@@ -323,21 +324,28 @@ class MoE(nn.Module):
         )
 
     def _compute_routing_weights(self, hidden_states: torch.Tensor):
-        """moe.py:246-257.  On the kernel path in eval mode the gate GEMM, top-k and softmax are one
-        kernel and the (T, E) logits are never written (only the training aux loss reads them)."""
-        if self._use_fused_router(hidden_states):
-            _, router_weights, selected_experts = ops.router_fused(
-                hidden_states, self.gate.weight, self.top_k, bias=self.router_logit_bias
-            )
-            return None, router_weights, selected_experts
+        """moe.py:246-257.  On the kernel path the gate GEMM, top-k and softmax are one kernel in every dtype; in
+        eval mode the (T, E) logits are never written (only the training aux loss and the backward read them); with
+        a gradient the same kernel runs inside autograd.FusedRouter, whose backward is kernels too."""
+        if (is_kernel_allowed(Kernel.scattermoe) and hidden_states.is_cuda
+                and ops.router_fused_supported(hidden_states, self.num_experts, self.top_k)):
+            if self._needs_grad(hidden_states):
+                return FusedRouter.apply(hidden_states, self.gate.weight, self.router_logit_bias, self.top_k)
+            return ops.router_fused(hidden_states, self.gate.weight, self.top_k, bias=self.router_logit_bias,
+                                    return_logits=self.training)
 
         router_logits = self.gate(hidden_states)
         if self.router_logit_bias is not None:
             router_logits = (router_logits.float() + self.router_logit_bias.float()).to(router_logits.dtype)
 
         if is_kernel_allowed(Kernel.scattermoe) and hidden_states.is_cuda:
-            # the kernel's tie rule (value descending, expert index ascending) in training and in inference alike:
-            # torch.topk documents no tie order, and bf16 logits tie often
+            # shapes the router kernel does not take (more than 256 experts, a hidden size that is not a multiple
+            # of 16): the logits come from torch, the selection still follows the kernel's tie rule (value
+            # descending, expert index ascending) in training and in inference alike
+            ops._warn_once(("router_unfused", self.num_experts, self.hidden_size, hidden_states.dtype),
+                           f"MoE router with {self.num_experts} experts, hidden size {self.hidden_size}, "
+                           f"{hidden_states.dtype}: not a shape of the fused router kernel; the logits are computed "
+                           "by torch's linear layer")
             with torch.no_grad():
                 router_weights, selected_experts = ops.router_topk_softmax(router_logits.detach(), self.top_k)
             if torch.is_grad_enabled() and router_logits.requires_grad:
@@ -424,18 +432,30 @@ class MoE(nn.Module):
         return hidden_states
 
     def _compute_shared_experts(self, hidden_states: torch.Tensor) -> torch.Tensor:
-        """moe.py:311-315.  On the kernel branch the dense SwiGLU MLP runs as a one-expert grouped GEMM (SwiGLU
-        in the up-projection's epilogue)."""
+        """moe.py:311-315.  On the kernel branch the dense MLP runs on the grouped-GEMM kernels as ONE expert that
+        owns every token (rows in place, no gather, no router weights): SwiGLU in the up-projection's epilogue in
+        inference, the differentiable forms of autograd.py when a gradient is needed; any of the three dtypes."""
         if (
-            is_kernel_allowed(Kernel.scattermoe) and self._fused_swiglu and hidden_states.is_cuda
+            is_kernel_allowed(Kernel.scattermoe) and hidden_states.is_cuda
             and self.c_fc_shared.bias is None and self.c_proj_shared.bias is None
-            and hidden_states.dtype in (torch.bfloat16, torch.float16) and not torch.is_grad_enabled()
+            and hidden_states.dtype in (torch.bfloat16, torch.float16, torch.float32)
         ):
             T = hidden_states.shape[0]
             rows = torch.arange(T, dtype=torch.int32, device=hidden_states.device)
             offsets = torch.full((1,), T, dtype=torch.int32, device=hidden_states.device)
-            act = ops.up_swiglu(hidden_states, self.c_fc_shared.weight.unsqueeze(0), 1, rows, offsets)
-            return ops.scattered_gemm(act, self.c_proj_shared.weight.unsqueeze(0), 1, rows, offsets, True, True)
+            w_fc, w_proj = self.c_fc_shared.weight.unsqueeze(0), self.c_proj_shared.weight.unsqueeze(0)
+            if self._fused_swiglu and self._needs_grad(hidden_states):
+                return ScatteredSwiGLUExperts.apply(hidden_states, w_fc, w_proj, None, rows, offsets, 1,
+                                                    self.keep_preactivation)
+            if self._fused_swiglu:
+                act = ops.up_swiglu(hidden_states, w_fc, 1, rows, offsets)
+                return ops.scattered_gemm(act, w_proj, 1, rows, offsets, True, True)
+            # any other activation: the two products through the (differentiable) drop-in op, torch in between
+            kw = dict(k=1, sorted_expert_idxs=None, sorted_scattered_idxs=rows, expert_offsets=offsets,
+                      grouped_in=True, grouped_out=True)
+            hidden_states = ops.scattered_experts(hidden_states, w_fc.permute(0, 2, 1), **kw)
+            hidden_states = self.act(hidden_states)
+            return ops.scattered_experts(hidden_states, w_proj.permute(0, 2, 1), **kw)
         hidden_states = self.c_fc_shared(hidden_states)
         hidden_states = self.act(hidden_states)
         hidden_states = self.c_proj_shared(hidden_states)

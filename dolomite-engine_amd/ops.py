@@ -130,8 +130,22 @@ def router_topk_softmax(logits: torch.Tensor, k: int) -> tuple[torch.Tensor, tor
     return gates, idx
 
 
-def router_fused_supported(x: torch.Tensor, num_experts: int, k: int) -> bool:
+def _router_streaming_supported(x: torch.Tensor, num_experts: int, k: int) -> bool:
+    """The streaming kernels of the fused router (gate weights in LDS, the split-K small-batch form, the forms with
+    the sort or the RMSNorm folded in): 16-bit, at most 64 experts, k <= 8."""
     return (x.dtype in (torch.bfloat16, torch.float16) and num_experts <= 64 and k <= 8 and x.shape[-1] % 16 == 0)
+
+
+def router_fused_supported(x: torch.Tensor, num_experts: int, k: int) -> bool:
+    """What :func:`router_fused` takes: the streaming kernels' shapes, and through the general kernel fp32
+    (H % 8 == 0), up to 256 experts and k up to 64 (16-bit: H % 16 == 0)."""
+    if _router_streaming_supported(x, num_experts, k):
+        return True
+    if not (1 <= k <= min(num_experts, 64) and num_experts <= 256):
+        return False
+    if x.dtype == torch.float32:
+        return x.shape[-1] % 8 == 0
+    return x.dtype in (torch.bfloat16, torch.float16) and x.shape[-1] % 16 == 0
 
 
 def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch.Tensor | None = None,
@@ -154,8 +168,9 @@ def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch
     gates = torch.empty((T, k), dtype=x.dtype, device=x.device)
     idx = torch.empty((T, k), dtype=torch.int32, device=x.device)
     lib = _lib.load()
-    # non-zero for few tokens: K split over the chip
-    ws_bytes = lib.mi_moe_router_fused_workspace_bytes(T, H, E) if split_k else 0
+    # non-zero for few tokens: K split over the chip (streaming kernels only)
+    ws_bytes = lib.mi_moe_router_fused_workspace_bytes(T, H, E) if (
+        split_k and _router_streaming_supported(x, E, k)) else 0
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
     with _stage("router_fused"):
         check(lib.mi_moe_router_fused(_ptr(x), _ptr(gate_weight), _ptr(bias), T, H, E, k, _code(x.dtype),
@@ -165,7 +180,7 @@ def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch
 
 def router_fused_sort_supported(x: torch.Tensor, num_experts: int, k: int) -> bool:
     """Small batches only (the split-K router and the one-block sort): T <= 1024 and T * k <= 8192."""
-    if not (router_fused_supported(x, num_experts, k) and x.is_cuda and x.dim() == 2 and x.shape[0] >= 1):
+    if not (_router_streaming_supported(x, num_experts, k) and x.is_cuda and x.dim() == 2 and x.shape[0] >= 1):
         return False
     return _lib.load().mi_moe_router_fused_sort_workspace_bytes(x.shape[0], x.shape[1], num_experts, k) > 0
 
@@ -236,6 +251,32 @@ def rmsnorm_router_fused(h: torch.Tensor, ln_weight: torch.Tensor | None, eps: f
                                                      T, H, E, k, _code(h.dtype), _ptr(x_norm), _ptr(logits),
                                                      _ptr(gates), _ptr(idx), _stream()))
     return x_norm, logits, gates, idx
+
+
+def router_dlogits(logits: torch.Tensor, experts: torch.Tensor, d_gates: torch.Tensor | None,
+                   d_logits_extra: torch.Tensor | None) -> torch.Tensor:
+    """Gradient of the router's outputs w.r.t. the (T, E) logits: the softmax over the k picked logits backwards,
+    scattered to the picked experts, plus ``d_logits_extra`` (the gradient that reaches the logits directly, i.e.
+    the auxiliary loss).  ``experts`` (T, k) int32, ``d_gates`` (T, k) or None, all floating tensors in
+    logits.dtype.  The element-wise part of the backward of moe.py:246-257."""
+    _dev(logits, experts, d_gates, d_logits_extra)
+    _no_grad(logits, d_gates, d_logits_extra)
+    logits = logits.contiguous()
+    experts = _i32(experts).contiguous()
+    T, E = logits.shape
+    k = experts.shape[1]
+    if experts.shape[0] != T:
+        raise ValueError("experts must be (T, k)")
+    for name, t, shape in (("d_gates", d_gates, (T, k)), ("d_logits_extra", d_logits_extra, (T, E))):
+        if t is not None and (tuple(t.shape) != shape or t.dtype != logits.dtype):
+            raise ValueError(f"{name} must be {shape} in the dtype of the logits")
+    d_gates = None if d_gates is None else d_gates.contiguous()
+    d_logits_extra = None if d_logits_extra is None else d_logits_extra.contiguous()
+    out = torch.empty_like(logits)
+    with _stage("router_dlogits"):
+        check(_lib.load().mi_moe_router_dlogits(_ptr(logits), _ptr(experts), _ptr(d_gates), _ptr(d_logits_extra), T, E, k,
+                                               _code(logits.dtype), _ptr(out), _stream()))
+    return out
 
 
 def continuous_count(x: torch.Tensor, size: int) -> torch.Tensor:

@@ -71,9 +71,12 @@ int mi_moe_router_topk_softmax(const void* logits, int T, int E, int k, int dtyp
  * Fused router: logits = x @ gate_w^T rounded to `dtype` (+ optional per-expert fp32 bias, rounded
  * again), then the top-k softmax above, in ONE pass over x.
  * Replaces: MoE._compute_routing_weights (moe.py:246-257).
- *   x (T, H), gate_w (E, H) of `dtype` (F16 / BF16), H % 8 == 0, E <= 64
+ *   x (T, H), gate_w (E, H) of `dtype`.  F16 / BF16 with E <= 64, k <= 8, H % 16 == 0 run the streaming
+ *   kernels (gate weights resident in LDS, x read once at HBM rate); F32 (H % 8 == 0), 65 .. 256 experts
+ *   and k up to 64 run a general kernel (one workgroup per 16 tokens) -- no shape of the layer needs a library
+ *   GEMM for its logits.  Anything else: MI_MOE_EUNSUPPORTED.
  *   bias       (E,) fp32 or NULL
- *   logits_out (T, E) of `dtype` or NULL (only the training-time aux loss reads it)
+ *   logits_out (T, E) of `dtype` or NULL (the training-time aux loss and the backward read it)
  *   ws / ws_bytes  optional scratch, 16-byte aligned.  With at least
  *                  mi_moe_router_fused_workspace_bytes(T, H, E) bytes (non-zero for T <= 1024) the
  *                  contraction is split over many workgroups and finished by a second small launch -- a few
@@ -83,6 +86,20 @@ size_t mi_moe_router_fused_workspace_bytes(int T, int H, int E);
 int mi_moe_router_fused(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,
                         int dtype, void* logits_out, void* gates_out, int32_t* idx_out, void* ws,
                         size_t ws_bytes, mi_moe_stream_t stream);
+
+/*
+ * Backward of the router's outputs w.r.t. its logits (the element-wise part of the gradient of
+ * MoE._compute_routing_weights, moe.py:246-257, which the reference leaves to autograd):
+ *   d_logits_out[t, e] = d_logits_extra[t, e] + (e == idx[t, j] ? p_j * (g_j - sum_i p_i g_i) : 0),
+ * p = fp32 softmax of the k picked logits, g = d_gates[t, :]; the picked term is rounded to `dtype` before the sum
+ * and the sum once more, as autograd's casts do on the eager branch.  d_gates (T, k) and d_logits_extra (T, E)
+ * (the gradient that reaches the logits directly: the auxiliary loss) may each be NULL (= zero).  The two
+ * products that complete the gradient -- d x = d_logits @ gate_w and d gate_w = d_logits^T @ x -- are
+ * mi_moe_scattered_gemm and mi_moe_grouped_wgrad called with one expert that owns every row.
+ *   logits (T, E), d_gates (T, k), d_logits_extra / d_logits_out (T, E) of `dtype` (F32 / F16 / BF16); k <= 64
+ */
+int mi_moe_router_dlogits(const void* logits, const int32_t* idx, const void* d_gates, const void* d_logits_extra,
+                          int T, int E, int k, int dtype, void* d_logits_out, mi_moe_stream_t stream);
 
 /*
  * Fused router followed by the expert sort / bin of mi_moe_sort_bin, for small batches (decode): the launch that

@@ -68,8 +68,17 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_router_topk_softmax(None, 4, 8, 9, _lib.BF16, None, None, None) == E_SHAPE  # k > E
     assert lib.mi_moe_router_topk_softmax(None, 4, 8, 2, _lib.BF16, None, None, None) == E_NULL
     assert lib.mi_moe_router_topk_softmax(None, 0, 8, 2, _lib.BF16, None, None, None) == 0  # empty input
-    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 128, 2, _lib.BF16, None, None, None, None, 0, None) == E_UNSUP
-    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 8, 2, _lib.F32, None, None, None, None, 0, None) == E_DTYPE
+    # fp32 and up to 256 experts are taken (general kernel); beyond that, or a ragged hidden size: refused
+    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 128, 2, _lib.BF16, None, None, None, None, 0, None) == E_NULL
+    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 8, 2, _lib.F32, None, None, None, None, 0, None) == E_NULL
+    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 300, 2, _lib.BF16, None, None, None, None, 0, None) == E_UNSUP
+    assert lib.mi_moe_router_fused(None, None, None, 4, 60, 8, 2, _lib.F32, None, None, None, None, 0, None) == E_UNSUP
+    assert lib.mi_moe_router_fused(None, None, None, 4, 72, 8, 2, _lib.BF16, None, None, None, None, 0, None) == E_UNSUP
+    assert lib.mi_moe_router_fused(None, None, None, 4, 64, 8, 2, 7, None, None, None, None, 0, None) == E_DTYPE
+    assert lib.mi_moe_router_dlogits(None, None, None, None, 4, 8, 9, _lib.BF16, None, None) == E_SHAPE
+    assert lib.mi_moe_router_dlogits(None, None, None, None, 4, 8, 2, 7, None, None) == E_DTYPE
+    assert lib.mi_moe_router_dlogits(None, None, None, None, 4, 8, 2, _lib.F32, None, None) == E_NULL
+    assert lib.mi_moe_router_dlogits(None, None, None, None, 0, 8, 2, _lib.F32, None, None) == 0
     assert lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) > 0
     assert lib.mi_moe_router_fused_workspace_bytes(32768, 1536, 40) == 0
     assert lib.mi_moe_router_fused_sort_workspace_bytes(64, 4096, 64, 6) == lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) + 256

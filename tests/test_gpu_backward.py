@@ -9,6 +9,8 @@ import pytest
 import torch
 import torch.nn.functional as F
 
+from _parity import assert_close_scaled
+
 pytestmark = pytest.mark.gpu
 
 
@@ -330,3 +332,36 @@ def test_grouped_wgrad_random_shapes(device, seed):
     got = _ops().grouped_wgrad(a.to(device), b.to(device), offsets.to(device), None, b_idx.to(device))
     ref = _wgrad_reference(a, b, offsets, None, b_idx)
     torch.testing.assert_close(got.cpu().double(), ref, rtol=2.0 ** -7, atol=2e-5 * max(1.0, counts.max().item()) ** 0.5 + 1e-6)
+
+
+@pytest.mark.parametrize("dtype,T,H,E,k", [(torch.bfloat16, 300, 128, 40, 8), (torch.float16, 257, 64, 136, 12),
+                                           (torch.float32, 100, 64, 8, 2), (torch.bfloat16, 2100, 1536, 40, 8)])
+def test_fused_router_function(device, dtype, T, H, E, k):
+    """autograd.FusedRouter (router kernel forward; d-logits kernel + grouped GEMM + grouped weight gradient
+    backward) against torch autograd through linear -> gather at the same experts -> float softmax -> cast
+    (moe.py:246-257), with gradients arriving at the gates and at the logits."""
+    from dolomite_engine_amd.autograd import FusedRouter
+
+    g = torch.Generator().manual_seed(T + E)
+    x0 = torch.randn(T, H, generator=g).to(dtype).to(device)
+    w0 = (torch.randn(E, H, generator=g) * 0.1).to(dtype).to(device)
+    dg = torch.randn(T, k, generator=g).to(dtype).to(device)
+    dl = (torch.randn(T, E, generator=g) * 0.05).to(dtype).to(device)
+    print(f"FusedRouter {dtype} T={T} H={H} E={E} k={k}", flush=True)
+
+    x, w = x0.clone().requires_grad_(True), w0.clone().requires_grad_(True)
+    logits, gates, experts = FusedRouter.apply(x, w, None, k)
+    ((gates * dg).sum() + (logits * dl).sum()).backward()
+
+    xr, wr = x0.clone().requires_grad_(True), w0.clone().requires_grad_(True)
+    logits_r = torch.nn.functional.linear(xr, wr)
+    gates_r = torch.softmax(logits_r.gather(-1, experts.long()).float(), dim=-1).to(dtype)
+    ((gates_r * dg).sum() + (logits_r * dl).sum()).backward()
+
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(logits.detach().float(), logits_r.detach().float(), **tol)
+    for name, got, want in (("dx", x.grad, xr.grad), ("dw", w.grad, wr.grad)):
+        scale = want.float().abs().max().clamp_min(1e-6)
+        assert_close_scaled(got, want, dtype, what=f"router {name}", rtol=tol["rtol"], atol=tol["atol"] * scale.item(),
+                            rel_to_max=2e-2 if dtype != torch.float32 else 1e-4,
+                            rel_rms_limit=1e-2 if dtype != torch.float32 else 1e-4)

@@ -148,6 +148,8 @@ def test_layer_edge_batches(device, dtype):
             flat = x_dev.reshape(-1, w.H)
             if flat.shape[0] and m._use_fused_router(flat) and ops.router_fused_sort_supported(flat, w.E, w.k):
                 logits = ops.router_fused_sort(flat, m.gate.weight, w.k, bias=m.router_logit_bias, return_logits=True)[0]
+            elif flat.shape[0] and ops.router_fused_supported(flat, w.E, w.k):
+                logits = ops.router_fused(flat, m.gate.weight, w.k, bias=m.router_logit_bias, return_logits=True)[0]
             else:
                 logits = m._compute_routing_weights(flat)[0]
         return y, logits
@@ -181,20 +183,34 @@ def test_layer_edge_batches(device, dtype):
     assert_close_scaled(yv, ref.y, dtype, what="edge non-contiguous", **tol)
 
 
-def test_layer_shared_experts(device):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_layer_shared_experts(device, dtype, monkeypatch):
+    """Shared experts (moe.py:311-315) on the kernel branch run on the grouped-GEMM kernels in every dtype: the
+    module's two shared linear layers must not be called at all."""
     from dolomite_engine_amd import Kernel, MoE, enable_kernels
 
     torch.manual_seed(7)
     m = MoE(hidden_size=128, intermediate_size=64, shared_intermediate_size=96, num_experts=8,
             num_experts_per_tok=2, activation_function="swiglu", add_bias=False, dropout=0.0, init_method="normal",
             initializer_range=0.05, m_width=None, num_layers=1, use_padding_free_transformer=True)
-    m = m.to(torch.bfloat16).to(device).eval()
-    x = torch.randn(300, 128, device=device, dtype=torch.bfloat16)
+    m = m.to(dtype).to(device).eval()
+    x = torch.randn(300, 128, device=device, dtype=dtype)
+
+    def refuse(*a, **k):
+        raise AssertionError("the shared experts went through torch's linear layer on the kernel branch")
+
+    monkeypatch.setattr(m.c_fc_shared, "forward", refuse)
+    monkeypatch.setattr(m.c_proj_shared, "forward", refuse)
     with torch.no_grad(), enable_kernels([Kernel.scattermoe]):
         y = m(x)
+        # the logits as the module's router kernel produced them (fp32 sums differ by order: route on these)
+        from dolomite_engine_amd import ops
+        logits = ops.router_fused(x, m.gate.weight, 2, return_logits=True)[0]
     ref = oracle.moe_forward(x.cpu(), m.gate.weight.cpu(), m.c_fc.weight.cpu(), m.c_proj.weight.cpu(), 2,
+                             logits=None if logits is None else logits.cpu(),
                              shared_fc=m.c_fc_shared.weight.cpu(), shared_proj=m.c_proj_shared.weight.cpu())
-    assert_close_scaled(y, ref.y, torch.bfloat16, rtol=2e-2, atol=2e-2, what="shared experts")
+    tol = dict(rtol=2e-2, atol=2e-2) if dtype == torch.bfloat16 else dict(rtol=1e-3, atol=2e-4)
+    assert_close_scaled(y, ref.y, dtype, what="shared experts", **tol)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -343,8 +359,6 @@ def test_training_gradients_match_eager_branch(device, dtype, tol, shared, activ
     # "swiglu": the pre-activation of the up-projection is kept for the backward; "swiglu-recompute": recomputed there
     keep = activation != "swiglu-recompute"
     activation = activation.split("-")[0]
-    if activation != "swiglu" and shared is not None:
-        pytest.skip("the shared experts do not depend on the routed experts' activation path")
     torch.manual_seed(21)
     m = MoE(hidden_size=128, intermediate_size=64, shared_intermediate_size=shared, num_experts=8,
             num_experts_per_tok=2, activation_function=activation, add_bias=False, dropout=0.0, init_method="normal",

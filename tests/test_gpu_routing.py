@@ -140,6 +140,93 @@ def test_router_fused(device, dtype, T, H, E, k, bias):
     assert ulp3 <= 1
 
 
+@pytest.mark.parametrize("dtype,T,H,E,k,bias", [
+    (torch.float32, 512, 256, 8, 2, False),      # the reference's correctness configuration
+    (torch.float32, 1, 8, 4, 1, False),
+    (torch.float32, 333, 136, 40, 8, True),
+    (torch.float32, 70, 1536, 200, 33, True),
+    (torch.bfloat16, 300, 256, 128, 8, True),    # more than 64 experts
+    (torch.float16, 129, 1024, 256, 64, False),  # k beyond the streaming kernels' 8
+    (torch.bfloat16, 50, 64, 40, 12, False),
+    (torch.bfloat16, 2100, 48, 65, 2, False),
+])
+def test_router_general(device, dtype, T, H, E, k, bias):
+    """fp32, more than 64 experts, k above 8: the general kernel behind the same entry point, held to the same
+    contract as the streaming kernels (logits = the oracle's up to the summation order, routing bit-exact on the
+    device's own logits, gates within one unit in the last place)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(T + H + E + k)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    w = (torch.randn(E, H, generator=g) * 0.05).to(dtype)
+    b = (torch.randn(E, generator=g) * 0.5) if bias else None
+    print(f"router general T={T} H={H} E={E} k={k} {dtype} bias={bias}", flush=True)
+    assert ops.router_fused_supported(x, E, k)
+    bd = None if b is None else b.to(device)
+    logits, gates, idx = ops.router_fused(x.to(device), w.to(device), k, bias=bd, return_logits=True)
+    logits = logits.cpu()
+    ref_logits = oracle.router_logits(x, w, b)
+    tol = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.bfloat16: dict(rtol=1.6e-2, atol=1e-3),
+           torch.float16: dict(rtol=2e-3, atol=1e-3)}[dtype]
+    torch.testing.assert_close(logits.float(), ref_logits.float(), **tol)
+    vals, ref_idx = oracle.topk_canonical(logits, k)
+    assert torch.equal(idx.cpu().long(), ref_idx)
+    ref_gates = oracle.softmax_topk(vals, dtype)
+    if dtype == torch.float32:
+        torch.testing.assert_close(gates.cpu(), ref_gates, rtol=1e-5, atol=1e-7)
+    else:
+        assert (gates.cpu().view(torch.int16).int() - ref_gates.view(torch.int16).int()).abs().max() <= 1
+    _, gates2, idx2 = ops.router_fused(x.to(device), w.to(device), k, bias=bd)
+    assert torch.equal(idx2, idx) and torch.equal(gates2, gates)
+
+
+def test_router_general_ties_and_special_values(device):
+    """Tie rule of the general kernel on logits built to tie: equal columns in the gate weight give equal logits
+    for every token; the lower expert index must win."""
+    ops = _ops()
+    T, H, E, k = 40, 64, 130, 5
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    base = (torch.randn(7, H, generator=g) * 0.1).to(torch.bfloat16)
+    w = base[torch.arange(E) % 7].contiguous()          # 130 experts, only 7 distinct rows: ties everywhere
+    logits, gates, idx = ops.router_fused(x.to(device), w.to(device), k, return_logits=True)
+    vals, ref_idx = oracle.topk_canonical(logits.cpu(), k)
+    assert torch.equal(idx.cpu().long(), ref_idx)
+    assert (gates.cpu().view(torch.int16).int() - oracle.softmax_topk(vals, torch.bfloat16).view(torch.int16).int()).abs().max() <= 1
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k", [(1, 4, 1), (15, 8, 8), (300, 40, 8), (129, 130, 2), (70, 256, 64)])
+@pytest.mark.parametrize("parts", ["gates", "extra", "both"])
+def test_router_dlogits(device, dtype, T, E, k, parts):
+    """d logits from (d gates, d logits_extra) against torch autograd through gather -> float softmax -> cast
+    (moe.py:250-255), in fp32 and rounded where autograd rounds."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(T * 7 + E + k)
+    logits = torch.randn(T, E, generator=g).to(dtype)
+    _, idx = oracle.topk_canonical(logits, k)
+    d_gates = torch.randn(T, k, generator=g).to(dtype) if parts != "extra" else None
+    extra = (torch.randn(T, E, generator=g) * 0.1).to(dtype) if parts != "gates" else None
+    got = ops.router_dlogits(logits.to(device), idx.to(torch.int32).to(device),
+                             None if d_gates is None else d_gates.to(device),
+                             None if extra is None else extra.to(device)).cpu()
+    lg = logits.clone().requires_grad_(True)
+    want = torch.zeros(T, E, dtype=dtype)
+    if d_gates is not None:
+        gates = torch.softmax(lg.gather(-1, idx).float(), dim=-1).to(dtype)
+        (gates * d_gates).sum().backward()
+        want = lg.grad
+    if extra is not None:
+        want = want + extra
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=0, atol=0)
+    if dtype != torch.float32:
+        # same fp32 arithmetic up to the order of the softmax's sum: a unit in the last place here and there
+        steps = (got.view(torch.int16).int() - want.view(torch.int16).int()).abs()
+        close = (got.float() - want.float()).abs() <= 1e-3 * want.float().abs() + 2e-6
+        assert bool(((steps <= 1) | close).all())
+    else:
+        torch.testing.assert_close(got, want, **tol)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,H,E,k,bias,gamma", [(1, 64, 8, 2, False, True), (200, 256, 40, 8, True, True),
                                                 (2500, 1536, 40, 8, True, True), (4099, 1024, 32, 8, False, False),
