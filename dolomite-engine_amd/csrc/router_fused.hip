@@ -75,11 +75,12 @@ __device__ __forceinline__ uint32_t router_max4(uint32_t x) {
 // Epilogue for one group of 16 tokens: lane (r = token, q) holds acc[eb][i] = logit of expert
 // 16*eb + 4*q + i.  Rounds to the model dtype, adds the optional bias, optionally stores the logits,
 // selects the top-k (value descending, expert ascending) and writes the softmax of the k winners.
+// `hist` (LDS, E counters shared by the workgroup, or null) receives one count per selected expert.
 template <typename T>
 __device__ __forceinline__ void router_epilogue(const f32x4 (&acc)[4], int t, bool tvalid, int q,
                                                 const float* __restrict__ bias, int E, int k,
                                                 T* __restrict__ logits_out, T* __restrict__ gates,
-                                                int32_t* __restrict__ idx) {
+                                                int32_t* __restrict__ idx, int* hist = nullptr) {
   uint32_t keys[16];
 #pragma unroll
   for (int eb = 0; eb < 4; ++eb) {
@@ -123,6 +124,7 @@ __device__ __forceinline__ void router_epilogue(const f32x4 (&acc)[4], int t, bo
       if (j < k) {
         Elt<T>::store(gates + (size_t)t * k + j, p[j] / denom);
         idx[(size_t)t * k + j] = wi[j];
+        if (hist != nullptr) atomicAdd(&hist[wi[j]], 1);
       }
     }
   }
@@ -222,10 +224,15 @@ struct RouterNorm {
   float eps;
 };
 
+// `chunk_hist` (or null): the first pass of the expert sort (routing.hip) done here.  The groups a workgroup takes
+// in one turn are consecutive -- a chunk of blockDim / 64 * 16 tokens -- so the workgroup counts the experts its
+// waves select in LDS and writes chunk_hist[e * nchunks + chunk], the layout the sort's scan pass reads; the sort
+// then needs neither its histogram launch nor that launch's read of the expert ids.
 template <typename T, int DEPTH, bool NORM>
 __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ gw, const float* __restrict__ bias, int Trows, int H, int E, int k,
-    T* __restrict__ logits_out, T* __restrict__ gates, int32_t* __restrict__ idx, RouterNorm norm) {
+    T* __restrict__ logits_out, T* __restrict__ gates, int32_t* __restrict__ idx, RouterNorm norm,
+    int32_t* __restrict__ chunk_hist, int nchunks) {
   typedef typename RMfma<T>::vec frag_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char wlds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -283,12 +290,15 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
     for (int i = 0; i < 8; ++i)
       if (dst[i] >= 0) *reinterpret_cast<u32x4*>(wlds + dst[i]) = v[i];
   }
-  // NORM: gamma (or ones) as fp32 behind the weights
+  // NORM: gamma (or ones) as fp32 behind the weights; then the E counters of the chunk histogram
   float* glds = reinterpret_cast<float*>(wlds + (size_t)E * pitch);
   if (NORM) {
     const T* gamma = static_cast<const T*>(norm.gamma);
     for (int i = threadIdx.x; i < H; i += blockDim.x) glds[i] = gamma != nullptr ? Elt<T>::load(gamma + i) : 1.0f;
   }
+  int* whist = reinterpret_cast<int*>(wlds + (size_t)E * pitch + (NORM ? (size_t)H * sizeof(float) : 0));
+  if (chunk_hist != nullptr)
+    for (int e = threadIdx.x; e < E; e += blockDim.x) whist[e] = 0;
   __syncthreads();
 
   const int neb = (E + 15) >> 4;
@@ -299,7 +309,10 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
     if (e > E - 1) e = E - 1;
     wbase[eb] = e * pitch;
   }
-  while (grp < ngroups) {
+  // with a histogram every wave walks the same number of turns (a turn ends in workgroup barriers)
+  const int nturns = chunk_hist != nullptr ? (ngroups + stride - 1) / stride : 0;
+  for (int turn = 0; chunk_hist != nullptr ? turn < nturns : grp < ngroups; ++turn) {
+    if (grp < ngroups) {
     float rstd = 1.0f;
     if (NORM) {
       // first pass over the group's rows: sum of squares of the 16 k this lane holds per step, then over the
@@ -377,7 +390,27 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
     const int t = grp * 16 + r;
     grp += stride;
     if (grp < ngroups) open_group(grp);
-    router_epilogue<T>(acc, t, t < Trows, q, bias, E, k, logits_out, gates, idx);
+    router_epilogue<T>(acc, t, t < Trows, q, bias, E, k, logits_out, gates, idx,
+                       chunk_hist != nullptr ? whist : nullptr);
+    } else {
+      grp += stride;
+    }
+    if (chunk_hist != nullptr) {
+      // all counts of this turn are in (LDS only: the x loads already in flight for the next turn stay in flight)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0), vmcnt / expcnt untouched
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      const int chunk = blockIdx.x + turn * gridDim.x;
+      for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        if (chunk < nchunks) chunk_hist[(size_t)e * nchunks + chunk] = whist[e];
+        whist[e] = 0;
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+    }
   }
 }
 
@@ -620,23 +653,33 @@ static int launch_router_splitk(const void* x, const void* gw, const float* bias
   return mi_launch_status();
 }
 
-template <typename T, bool NORM>
-static int launch_router_lds(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
-                             void* logits_out, void* gates, int32_t* idx, RouterNorm norm, size_t lds, hipStream_t s) {
+// launch shape of the LDS-resident kernel: workgroups and waves per workgroup
+static int router_lds_shape(int T_, int* blocks, int* waves) {
   int cus = 0;
-  int rc = mi_cu_count(&cus);
+  const int rc = mi_cu_count(&cus);
   if (rc != MI_MOE_OK) return rc;
   const int groups = mi_ceil_div(T_, 16);
-  const int blocks = groups < cus ? groups : cus;
-  int waves = mi_ceil_div(groups, blocks);
-  if (waves > ROUTER_LDS_WAVES) waves = ROUTER_LDS_WAVES;
+  *blocks = groups < cus ? groups : cus;
+  int w = mi_ceil_div(groups, *blocks);
+  *waves = w > ROUTER_LDS_WAVES ? ROUTER_LDS_WAVES : w;
+  return MI_MOE_OK;
+}
+
+// `lds`: gate weights (+ gamma); the E counters of the chunk histogram come on top
+template <typename T, bool NORM>
+static int launch_router_lds(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
+                             void* logits_out, void* gates, int32_t* idx, RouterNorm norm, size_t lds, hipStream_t s,
+                             int32_t* chunk_hist = nullptr, int nchunks = 0) {
+  int blocks = 0, waves = 0;
+  int rc = router_lds_shape(T_, &blocks, &waves);
+  if (rc != MI_MOE_OK) return rc;
   auto kern = waves > 4 ? router_fused_lds_kernel<T, 3, NORM> : router_fused_lds_kernel<T, 6, NORM>;
   static std::atomic<uint64_t> lds_ok[2];  // the LDS size varies with E and H: opt in to the most it can be
   rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok[waves > 4 ? 1 : 0]);
   if (rc != MI_MOE_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(waves * 64), lds, s, static_cast<const T*>(x),
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(waves * 64), lds + (size_t)E * sizeof(int), s, static_cast<const T*>(x),
                      static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out),
-                     static_cast<T*>(gates), idx, norm);
+                     static_cast<T*>(gates), idx, norm, chunk_hist, nchunks);
   return mi_launch_status();
 }
 
@@ -691,9 +734,28 @@ static int launch_router_splitk_sort(const void* x, const void* gw, const float*
   return mi_launch_status();
 }
 
+// Many tokens: router (LDS-resident gate weights) with the sort's histogram pass folded in, then the sort's scan
+// and scatter passes (routing.hip) on chunks of waves * 16 tokens.
+int mi_sort_after_hist(const int32_t* topk_idx, int L, int E, int chunk, int32_t* sorted_expert,
+                       int32_t* sorted_scattered, int32_t* expert_offsets, int32_t* ws, hipStream_t s);
+
+static bool router_hist_shape(int T_, int H, int E, int k, int* chunk_tokens, int* nchunks) {
+  if (T_ <= 1024 || (long)T_ * k > 0x7fffffffL - 8192) return false;
+  if ((size_t)E * ((size_t)H * 2 + 16) > 156u * 1024u) return false;  // gate weights must fit in LDS
+  int blocks = 0, waves = 0;
+  if (router_lds_shape(T_, &blocks, &waves) != MI_MOE_OK) return false;
+  *chunk_tokens = waves * 16;
+  *nchunks = mi_ceil_div(T_, *chunk_tokens);
+  return true;
+}
+
 extern "C" size_t mi_moe_router_fused_sort_workspace_bytes(int T, int H, int E, int k) {
-  (void)E;
-  return (T < 1 || H < 1 || k < 1) ? 0 : router_sort_ws_bytes(T, H, k);
+  if (T < 1 || H < 1 || k < 1 || E < 1) return 0;
+  const size_t small = router_sort_ws_bytes(T, H, k);
+  if (small) return small;
+  int chunk_tokens = 0, nchunks = 0;
+  if (E > 64 || k > ROUTER_KMAX || H % 16 != 0 || !router_hist_shape(T, H, E, k, &chunk_tokens, &nchunks)) return 0;
+  return ((size_t)E * nchunks + (size_t)E) * sizeof(int32_t);
 }
 
 extern "C" int mi_moe_router_fused_sort(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,
@@ -703,17 +765,31 @@ extern "C" int mi_moe_router_fused_sort(const void* x, const void* gate_w, const
   if (T < 1 || H < 1 || E < 1 || k < 1 || k > E) return MI_MOE_ESHAPE;
   if (E > 64 || k > ROUTER_KMAX || H % 16 != 0) return MI_MOE_EUNSUPPORTED;
   if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
-  const size_t need = router_sort_ws_bytes(T, H, k);
-  if (need == 0) return MI_MOE_EUNSUPPORTED;  // too many tokens for the split-K router or the one-block sort
+  const size_t need = mi_moe_router_fused_sort_workspace_bytes(T, H, E, k);
+  if (need == 0) return MI_MOE_EUNSUPPORTED;  // neither the few-token form nor the LDS-resident form takes the shape
   if (!x || !gate_w || !gates_out || !idx_out || !sorted_expert || !sorted_scattered || !expert_offsets) return MI_MOE_ENULL;
   if (!ws || ws_bytes < need) return MI_MOE_EWORKSPACE;
   if (!mi_aligned(x, 16) || !mi_aligned(gate_w, 16) || !mi_aligned(ws, 16)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == MI_MOE_BF16)
-    return launch_router_splitk_sort<bf16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, sorted_expert,
-                                             sorted_scattered, expert_offsets, ws, s);
-  return launch_router_splitk_sort<f16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, sorted_expert,
-                                          sorted_scattered, expert_offsets, ws, s);
+  if (router_sort_ws_bytes(T, H, k) != 0) {
+    if (dtype == MI_MOE_BF16)
+      return launch_router_splitk_sort<bf16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out,
+                                               sorted_expert, sorted_scattered, expert_offsets, ws, s);
+    return launch_router_splitk_sort<f16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out, sorted_expert,
+                                            sorted_scattered, expert_offsets, ws, s);
+  }
+  int chunk_tokens = 0, nchunks = 0;
+  router_hist_shape(T, H, E, k, &chunk_tokens, &nchunks);
+  const RouterNorm none = {nullptr, nullptr, 0.f};
+  const size_t wbytes = (size_t)E * ((size_t)H * 2 + 16);
+  int32_t* hist = static_cast<int32_t*>(ws);
+  const int rc = dtype == MI_MOE_BF16
+                     ? launch_router_lds<bf16_t, false>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out,
+                                                        none, wbytes, s, hist, nchunks)
+                     : launch_router_lds<f16_t, false>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out,
+                                                       none, wbytes, s, hist, nchunks);
+  if (rc != MI_MOE_OK) return rc;
+  return mi_sort_after_hist(idx_out, T * k, E, chunk_tokens * k, sorted_expert, sorted_scattered, expert_offsets, hist, s);
 }
 
 extern "C" size_t mi_moe_router_fused_workspace_bytes(int T, int H, int E) {

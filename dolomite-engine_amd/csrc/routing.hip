@@ -104,9 +104,9 @@ extern "C" int mi_moe_count(const int32_t* ids, int L, int E, uint32_t* counts_o
 //
 // The L slots are cut into chunks of SORT_CHUNK consecutive slots, one block per chunk.
 //   pass 1  per-chunk histogram in LDS                   -> ws[e * nblk + b]
-//   pass 2  per expert: exclusive scan over the chunks (in place); scan over the experts gives the
-//           inclusive expert_offsets (output) and the exclusive expert bases (ws tail)
-//   pass 3  each chunk is re-read in order; wave w of the block owns a contiguous quarter of the
+//   pass 2  per expert: exclusive scan over the chunks (in place) and the expert's total (ws tail)
+//   pass 3  every block scans the expert totals (expert bases; block 0 writes the inclusive expert_offsets);
+//           each chunk is re-read in order; wave w of the block owns a contiguous quarter of the
 //           chunk and walks it 64 slots at a time, so "earlier slot" == "earlier wave, earlier step,
 //           lower lane" and ranks come from a match-any ballot: the scatter is stable.
 // Small inputs (one chunk) run all three passes inside a single block and need no workspace.
@@ -129,55 +129,79 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_hist_kernel(const int32_t* 
   for (int e = threadIdx.x; e < E; e += SORT_THREADS) ws[(size_t)e * nblk + blockIdx.x] = hist[e];
 }
 
-// single block of 1024 threads (16 waves)
-__global__ __launch_bounds__(1024) void sort_scan_kernel(int E, int nblk, int32_t* __restrict__ ws,
-                                                         int32_t* __restrict__ expert_offsets) {
-  __shared__ int totals[SORT_MAX_E];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int e = wave; e < E; e += 16) {
-    int32_t* row = ws + (size_t)e * nblk;
-    int carry = 0;
-    for (int b0 = 0; b0 < nblk; b0 += 64) {
-      int b = b0 + lane;
-      int v = b < nblk ? row[b] : 0;
-      int inc = wave_incl_scan_i32(v, lane);
-      if (b < nblk) row[b] = carry + inc - v;
-      carry += __shfl(inc, 63, MI_WAVE);
-    }
-    if (lane == 0) totals[e] = carry;
+// Pass 2: one wave per expert (16 per block, ceil(E / 16) blocks).  Lane l owns the chunks [l * C, (l + 1) * C),
+// C = ceil(nblk / 64): its loads are all in flight at once (a walk along the row 64 chunks at a time pays one
+// memory latency per step), the lane totals are scanned across the wave and the exclusive prefixes written back in
+// place.  The expert's total goes to ws[E * nblk + e]; the scan over the experts is left to pass 3, so that no
+// block here waits for another.
+#define SORT_SCAN_BATCH 8
+__global__ __launch_bounds__(1024) void sort_scan_kernel(int E, int nblk, int32_t* __restrict__ ws) {
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.x * 16 + (threadIdx.x >> 6);
+  if (e >= E) return;
+  int32_t* row = ws + (size_t)e * nblk;
+  const int C = (nblk + 63) >> 6;
+  const int begin = lane * C;
+  int end = begin + C;
+  if (end > nblk) end = nblk;
+  // lane total (batches of independent loads)
+  int total = 0;
+  for (int b0 = begin; b0 < end; b0 += SORT_SCAN_BATCH) {
+    int v[SORT_SCAN_BATCH];
+#pragma unroll
+    for (int i = 0; i < SORT_SCAN_BATCH; ++i) v[i] = b0 + i < end ? row[b0 + i] : 0;
+#pragma unroll
+    for (int i = 0; i < SORT_SCAN_BATCH; ++i) total += v[i];
   }
-  __syncthreads();
-  if (wave == 0) {
+  const int incl = wave_incl_scan_i32(total, lane);
+  int run = incl - total;  // slots of this expert in the chunks before this lane's
+  for (int b0 = begin; b0 < end; b0 += SORT_SCAN_BATCH) {
+    int v[SORT_SCAN_BATCH];
+#pragma unroll
+    for (int i = 0; i < SORT_SCAN_BATCH; ++i) v[i] = b0 + i < end ? row[b0 + i] : 0;  // (cached: just read)
+#pragma unroll
+    for (int i = 0; i < SORT_SCAN_BATCH; ++i) {
+      if (b0 + i < end) row[b0 + i] = run;
+      run += v[i];
+    }
+  }
+  if (lane == 63) ws[(size_t)E * nblk + e] = incl;
+}
+
+// `chunk`: slots per block (SORT_CHUNK, or what one workgroup of the fused router counted in one turn).  Every block
+// scans the E expert totals itself (first wave) to get the experts' first output positions; block 0 also writes the
+// inclusive expert_offsets.
+__global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(const int32_t* __restrict__ ids, int L, int E,
+                                                                    int nbits, int nblk, int chunk,
+                                                                    const int32_t* __restrict__ ws,
+                                                                    int32_t* __restrict__ sorted_expert,
+                                                                    int32_t* __restrict__ sorted_scattered,
+                                                                    int32_t* __restrict__ expert_offsets) {
+  extern __shared__ int wcnt[];  // SORT_WAVES * E counters, then E expert bases
+  int* ebase = wcnt + SORT_WAVES * E;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < SORT_WAVES * E; i += SORT_THREADS) wcnt[i] = 0;
+  if (wave == SORT_WAVES - 1) {  // (the last wave: the others start on the histogram meanwhile)
+    const int32_t* totals = ws + (size_t)E * nblk;
     int carry = 0;
-    int32_t* ebase = ws + (size_t)E * nblk;
     for (int e0 = 0; e0 < E; e0 += 64) {
-      int e = e0 + lane;
-      int v = e < E ? totals[e] : 0;
-      int inc = wave_incl_scan_i32(v, lane);
+      const int e = e0 + lane;
+      const int v = e < E ? totals[e] : 0;
+      const int inc = wave_incl_scan_i32(v, lane);
       if (e < E) {
-        expert_offsets[e] = carry + inc;
         ebase[e] = carry + inc - v;
+        if (blockIdx.x == 0) expert_offsets[e] = carry + inc;
       }
       carry += __shfl(inc, 63, MI_WAVE);
     }
   }
-}
-
-__global__ __launch_bounds__(SORT_THREADS) void sort_scatter_kernel(const int32_t* __restrict__ ids, int L, int E,
-                                                                    int nbits, int nblk,
-                                                                    const int32_t* __restrict__ ws,
-                                                                    int32_t* __restrict__ sorted_expert,
-                                                                    int32_t* __restrict__ sorted_scattered) {
-  extern __shared__ int wcnt[];  // SORT_WAVES * E
-  for (int i = threadIdx.x; i < SORT_WAVES * E; i += SORT_THREADS) wcnt[i] = 0;
   __syncthreads();
-  const int chunk_begin = blockIdx.x * SORT_CHUNK;
-  int chunk_end = chunk_begin + SORT_CHUNK;
+  const int chunk_begin = blockIdx.x * chunk;
+  int chunk_end = chunk_begin + chunk;
   if (chunk_end > L) chunk_end = L;
-  const int per_wave = SORT_CHUNK / SORT_WAVES;
+  const int per_wave = (chunk + SORT_WAVES - 1) / SORT_WAVES;
   sort_wave_hist(ids, chunk_begin, chunk_end, per_wave, E, wcnt);
   __syncthreads();
-  const int32_t* ebase = ws + (size_t)E * nblk;
   for (int e = threadIdx.x; e < E; e += SORT_THREADS) {
     int run = ws[(size_t)e * nblk + blockIdx.x] + ebase[e];
 #pragma unroll
@@ -230,10 +254,25 @@ extern "C" int mi_moe_sort_bin(const int32_t* topk_idx, int T, int k, int E, int
   if (!mi_aligned(ws, 16)) return MI_MOE_EALIGN;
   int32_t* w = static_cast<int32_t*>(ws);
   hipLaunchKernelGGL(sort_hist_kernel, dim3(nblk), dim3(SORT_THREADS), 0, s, topk_idx, L, E, nblk, w);
-  hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(1024), 0, s, E, nblk, w, expert_offsets);
-  size_t lds = (size_t)SORT_WAVES * E * sizeof(int);
-  hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblk), dim3(SORT_THREADS), lds, s, topk_idx, L, E, nbits, nblk, w,
-                     sorted_expert, sorted_scattered);
+  hipLaunchKernelGGL(sort_scan_kernel, dim3(mi_ceil_div(E, 16)), dim3(1024), 0, s, E, nblk, w);
+  size_t lds = (size_t)(SORT_WAVES + 1) * E * sizeof(int);
+  hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblk), dim3(SORT_THREADS), lds, s, topk_idx, L, E, nbits, nblk,
+                     SORT_CHUNK, w, sorted_expert, sorted_scattered, expert_offsets);
+  return mi_launch_status();
+}
+
+// Passes 2 and 3 alone, for a caller that has produced pass 1 itself: the fused router (router_fused.hip) writes
+// ws[e * nblk + b] = number of slots of chunk b that go to expert e, chunks of `chunk` consecutive slots, nblk =
+// ceil(L / chunk); ws has room for E more words behind the histograms.  Arguments are validated by the caller.
+int mi_sort_after_hist(const int32_t* topk_idx, int L, int E, int chunk, int32_t* sorted_expert,
+                       int32_t* sorted_scattered, int32_t* expert_offsets, int32_t* ws, hipStream_t s) {
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  const int nblk = mi_ceil_div(L, chunk);
+  hipLaunchKernelGGL(sort_scan_kernel, dim3(mi_ceil_div(E, 16)), dim3(1024), 0, s, E, nblk, ws);
+  const size_t lds = (size_t)(SORT_WAVES + 1) * E * sizeof(int);
+  hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblk), dim3(SORT_THREADS), lds, s, topk_idx, L, E, nbits, nblk, chunk, ws,
+                     sorted_expert, sorted_scattered, expert_offsets);
   return mi_launch_status();
 }
 

@@ -102,12 +102,17 @@ int mi_moe_router_dlogits(const void* logits, const int32_t* idx, const void* d_
                           int T, int E, int k, int dtype, void* d_logits_out, mi_moe_stream_t stream);
 
 /*
- * Fused router followed by the expert sort / bin of mi_moe_sort_bin, for small batches (decode): the launch that
- * finishes the router also sorts (its last workgroup to finish does), one launch boundary less in a chain of short
- * dependent launches.  Replaces: MoE._compute_routing_weights + the sort / bincount / cumsum of the scatter branch
- * (moe.py:246-257, 263-271).  Same outputs as the two separate calls, bit for bit.
- * Taken when mi_moe_router_fused_sort_workspace_bytes(T, H, E, k) is non-zero: T <= 1024 and T * k <= 8192 (and the
- * limits of mi_moe_router_fused); MI_MOE_EUNSUPPORTED otherwise.  ws: that many bytes, 16-byte aligned.
+ * Fused router followed by the expert sort / bin of mi_moe_sort_bin, with the seam between them removed.
+ * Replaces: MoE._compute_routing_weights + the sort / bincount / cumsum of the scatter branch
+ * (moe.py:246-257, 263-271).  Same outputs as the two separate calls, bit for bit.  Two forms:
+ *   few tokens (T <= 1024 and T * k <= 8192; decode): the launch that finishes the split-K router also sorts (its
+ *     last workgroup to finish does) -- two launches instead of three in a chain of short dependent launches;
+ *   many tokens, gate weights resident in LDS (E * (2 H + 16) <= 156 KiB): the router's epilogue counts the
+ *     selected experts per chunk of consecutive tokens (the sort's first pass, without a launch of its own or a
+ *     second read of the expert ids), then the sort's scan and scatter passes run -- three launches instead of four.
+ * Taken when mi_moe_router_fused_sort_workspace_bytes(T, H, E, k) is non-zero (F16 / BF16, E <= 64, k <= 8,
+ * H % 16 == 0 and one of the two forms; the size depends on the device's compute-unit count, 0 without a device);
+ * MI_MOE_EUNSUPPORTED otherwise.  ws: that many bytes, 16-byte aligned.
  */
 size_t mi_moe_router_fused_sort_workspace_bytes(int T, int H, int E, int k);
 int mi_moe_router_fused_sort(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,

@@ -82,9 +82,9 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) > 0
     assert lib.mi_moe_router_fused_workspace_bytes(32768, 1536, 40) == 0
     assert lib.mi_moe_router_fused_sort_workspace_bytes(64, 4096, 64, 6) == lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) + 256
-    assert lib.mi_moe_router_fused_sort_workspace_bytes(2048, 1024, 32, 8) == 0   # too many tokens
+    assert lib.mi_moe_router_fused_sort_workspace_bytes(2048, 4096, 64, 8) == 0   # many tokens, gate weights beyond LDS
     assert lib.mi_moe_router_fused_sort_workspace_bytes(1024, 1024, 64, 9) == 0   # T * k beyond the one-block sort
-    assert lib.mi_moe_router_fused_sort(None, None, None, 2048, 1024, 32, 8, _lib.BF16, None, None, None, None, None,
+    assert lib.mi_moe_router_fused_sort(None, None, None, 2048, 4096, 64, 8, _lib.BF16, None, None, None, None, None,
                                         None, None, 0, None) == E_UNSUP
     assert lib.mi_moe_router_fused_sort(None, None, None, 64, 4096, 64, 6, _lib.BF16, None, None, None, None, None,
                                         None, None, 0, None) == E_NULL

@@ -276,11 +276,16 @@ def test_rmsnorm_router_fused_unsupported_shapes(device):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,H,E,k,bias", [(1, 64, 8, 2, False), (15, 32, 8, 8, False), (64, 4096, 64, 6, False),
                                           (200, 256, 40, 8, True), (1000, 1024, 32, 8, False), (1024, 512, 64, 8, True),
-                                          (130, 48, 5, 1, False)])
+                                          (130, 48, 5, 1, False),
+                                          # many tokens: the router counts the experts per chunk for the sort
+                                          (1025, 64, 8, 2, False), (2500, 256, 40, 8, True), (4099, 512, 64, 6, False),
+                                          (16384, 1024, 32, 8, False), (32768, 1536, 40, 8, True),
+                                          (70001, 128, 40, 1, False), (40000, 256, 16, 3, True)])
 def test_router_fused_sort_equals_separate_calls(device, dtype, T, H, E, k, bias):
-    """Small batches: the router launch that also sorts must give exactly what the fused router followed by
-    mi_moe_sort_bin gives -- logits, gates, experts, sorted order, offsets -- and the sort must be the oracle's.
-    Called twice, so that a ticket counter left over from the first call would show."""
+    """The router call that also sorts -- few tokens: its finishing launch sorts; many tokens: its epilogue counts
+    the experts per chunk and the sort's scan and scatter passes follow -- must give exactly what the fused router
+    followed by mi_moe_sort_bin gives (logits, gates, experts, sorted order, offsets), and the sort must be the
+    oracle's.  Called twice, so that a counter left over from the first call would show."""
     ops = _ops()
     g = torch.Generator().manual_seed(T * 7 + H + E)
     x = torch.randn(T, H, generator=g).to(dtype).to(device)
@@ -302,6 +307,7 @@ def test_router_fused_sort_equals_separate_calls(device, dtype, T, H, E, k, bias
 def test_router_fused_sort_limits(device):
     ops = _ops()
     x = torch.zeros(2048, 64, dtype=torch.bfloat16, device=device)
-    assert not ops.router_fused_sort_supported(x, 8, 2)          # more than 1024 tokens
+    assert ops.router_fused_sort_supported(x, 8, 2)              # many tokens: the form that counts per chunk
+    assert not ops.router_fused_sort_supported(torch.zeros(2048, 4096, dtype=torch.bfloat16, device=device), 64, 2)  # gate weights beyond LDS
     assert not ops.router_fused_sort_supported(x[:1024], 64, 9)  # k beyond the fused router
     assert ops.router_fused_sort_supported(x[:1024], 64, 8)      # 8192 slots: the one-block sort's limit
