@@ -56,7 +56,7 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
         E, I2, _ = w_fc.shape
         I = I2 // 2
         dy = dy.contiguous()
-        half = x.dtype in (torch.float16, torch.bfloat16) and I % 8 == 0
+        half = ops.elementwise_supported(x.dtype, I)  # (else: a ragged intermediate size, torch arithmetic)
 
         # gradient w.r.t. the SwiGLU output a, in sorted order and before the router weight: dy[t_i] @ w_proj[e_i]
         d_act = ops.scattered_gemm(dy, w_proj, k, ss, off, False, True, weight_kn=True)
@@ -88,12 +88,8 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
 
         # gradient w.r.t. x: every slot's contribution in flat-slot order, then the k slots of a token summed
         dx_slots = ops.scattered_gemm(d_h, w_fc, 1, ss, off, True, False, weight_kn=True)
-        if k == 1:
-            dx = dx_slots
-        elif half:
-            dx = ops.combine(dx_slots, torch.ones((T, k), dtype=x.dtype, device=x.device))
-        else:
-            dx = dx_slots.view(T, k, H).sum(dim=1)
+        # (the k slots of a token summed in slot order by the combine kernel with unit gates)
+        dx = dx_slots if k == 1 else ops.combine(dx_slots, torch.ones((T, k), dtype=x.dtype, device=x.device))
         del dx_slots
 
         # weight gradients: per expert X^T dY over that expert's rows
@@ -131,7 +127,6 @@ class ScatteredExperts(torch.autograd.Function):
         E, N, K = w.shape
         L = ss.numel()
         d_out = d_out.contiguous()
-        half = x.dtype in (torch.float16, torch.bfloat16)
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
 
         d_gates = None
@@ -139,7 +134,7 @@ class ScatteredExperts(torch.autograd.Function):
             T, kg = gates.shape
             if ctx.needs_input_grad[5]:
                 rows = ops.scattered_gemm(x, w, k, ss, off, grouped_in, False)
-                if half and N % 8 == 0:
+                if ops.elementwise_supported(rows.dtype, N):
                     d_gates = ops.combine_grad_gates(rows, d_out, kg).to(gates.dtype)
                 else:
                     d_gates = torch.bmm(rows.view(T, kg, N), d_out.unsqueeze(-1)).squeeze(-1).to(gates.dtype)
@@ -152,8 +147,7 @@ class ScatteredExperts(torch.autograd.Function):
             # row i: d_out[orow(i)] @ w[e_i], delivered to irow(i) (kept per slot first when a token fans out to k)
             dx = ops.scattered_gemm(d_out, w, 1, ss, off, grouped_out, grouped_in, weight_kn=True)
             if not grouped_in and k > 1:
-                dx = ops.combine(dx, torch.ones((L // k, k), dtype=dx.dtype, device=dx.device)) if half \
-                    else dx.view(L // k, k, K).sum(dim=1)
+                dx = ops.combine(dx, torch.ones((L // k, k), dtype=dx.dtype, device=dx.device))
 
         dw = None
         if need_w:

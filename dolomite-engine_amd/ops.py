@@ -453,9 +453,17 @@ def combine(o: torch.Tensor, gates: torch.Tensor, shared: torch.Tensor | None = 
     return y
 
 
+def elementwise_supported(dtype: torch.dtype, row_length: int) -> bool:
+    """Shapes the element-wise forward / backward kernels take: rows of whole 16-byte chunks."""
+    if dtype == torch.float32:
+        return row_length % 4 == 0
+    return dtype in (torch.float16, torch.bfloat16) and row_length % 8 == 0
+
+
 def swiglu_forward(h: torch.Tensor) -> torch.Tensor:
     """``h[:, :I] * silu(h[:, I:])`` for a stored pre-activation h (L, 2I) (activations/glu.py:42-43): fp32
-    arithmetic on the rounded h, one rounding.  16-bit dtypes with I % 8 == 0 run the kernel, anything else torch."""
+    arithmetic on the rounded h, one rounding.  Rows of whole 16-byte chunks (I % 8 == 0; fp32: I % 4 == 0) run the
+    kernel, a ragged I runs torch."""
     _dev(h)
     _no_grad(h)
     h = h.contiguous()
@@ -463,7 +471,7 @@ def swiglu_forward(h: torch.Tensor) -> torch.Tensor:
     I = I2 // 2
     if I2 % 2:
         raise ValueError("h must be (L, 2I)")
-    if h.dtype not in (torch.float16, torch.bfloat16) or I % 8:
+    if not elementwise_supported(h.dtype, I):
         up, gate = h[:, :I].float(), h[:, I:].float()
         return (up * gate * torch.sigmoid(gate)).to(h.dtype)
     act = torch.empty((L, I), dtype=h.dtype, device=h.device)
@@ -480,7 +488,7 @@ def swiglu_backward(h: torch.Tensor, d_act: torch.Tensor, gates: torch.Tensor | 
     ``d_act`` (L, I) is the gradient w.r.t. ``a`` before the router weight; row i is scaled by
     ``g_i = gates.flatten()[sorted_scattered_idxs[i]]`` (1 without ``gates``).  Returns ``(d_h, act_g, d_gates)``:
     ``d_h`` (L, 2I); ``act_g = g * a`` (L, I) if ``want_act``; ``d_gates`` in the shape of ``gates`` with
-    ``<d_act[i], a[i]>`` at the slot of row i if ``want_gate_grad``.  16-bit dtypes."""
+    ``<d_act[i], a[i]>`` at the slot of row i if ``want_gate_grad``.  Shapes: :func:`elementwise_supported`."""
     _dev(h, d_act, gates, sorted_scattered_idxs)
     _no_grad(h, d_act)
     h = h.contiguous()
@@ -509,7 +517,8 @@ def swiglu_backward(h: torch.Tensor, d_act: torch.Tensor, gates: torch.Tensor | 
 
 
 def combine_grad_gates(o: torch.Tensor, dy: torch.Tensor, k: int) -> torch.Tensor:
-    """d_gates[t, j] = <dy[t], o[t*k + j]>: the gradient of :func:`combine` w.r.t. the gates.  16-bit dtypes."""
+    """d_gates[t, j] = <dy[t], o[t*k + j]>: the gradient of :func:`combine` w.r.t. the gates.  Shapes:
+    :func:`elementwise_supported`."""
     _dev(o, dy)
     _no_grad(o, dy)
     o = o.contiguous()

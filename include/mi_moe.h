@@ -282,7 +282,8 @@ int mi_moe_combine_block_tail(const void* o, const void* gates, const void* shar
 /*
  * Element-wise pieces of the backward pass (training through the kernel branch).  The reference gets its
  * gradients from the autograd function of the external scattermoe package (moe.py:91-101); these two are
- * the parts of that backward that are neither a grouped GEMM nor a library GEMM.  F16 / BF16 only.
+ * the parts of that backward that are neither a grouped GEMM nor a library GEMM.  F32 / F16 / BF16; row lengths
+ * are whole 16-byte chunks (a multiple of 8 values of a 16-bit type, of 4 for F32).
  *
  * mi_moe_swiglu_backward, one pass over the sorted rows i = 0..L-1:
  *   h (L, 2I) = [up | gate] pre-activation, d_act (L, I) = gradient w.r.t. a = up * silu(gate)
@@ -291,16 +292,16 @@ int mi_moe_combine_block_tail(const void* o, const void* gates, const void* shar
  *   d_h (L, 2I) out = [g d_act * silu(gate) | g d_act * up * silu'(gate)]
  *   act_g (L, I) out or NULL = g * a               (operand of the down-projection's weight gradient)
  *   d_gates (T*k) out or NULL: d_gates[slot(i)] = <d_act[i], a[i]>   (= <dy[t], w_proj[e] a>, gradient of the
- *   router weight; every slot is written exactly once).  I % 8 == 0.
+ *   router weight; every slot is written exactly once).  I % 8 == 0 (F32: I % 4 == 0).
  */
 int mi_moe_swiglu_backward(const void* h, const void* d_act, const void* gates, const int32_t* sorted_scattered,
                            void* d_h, void* act_g, void* d_gates, int L, int I, int dtype, mi_moe_stream_t stream);
 /* The activation on its own, act_out (L, I) = h[:, :I] * silu(h[:, I:]) for a stored pre-activation h (L, 2I):
  * the GLUActivation the reference applies to the output of the up-projection (moe.py:281, glu.py:42-43).  A
  * training step that keeps h for the backward uses the unfused pair (mi_moe_scattered_gemm, this) in place of
- * mi_moe_up_swiglu.  I % 8 == 0. */
+ * mi_moe_up_swiglu.  I % 8 == 0 (F32: I % 4 == 0). */
 int mi_moe_swiglu_forward(const void* h, void* act_out, int L, int I, int dtype, mi_moe_stream_t stream);
-/* d_gates[t, j] = <dy[t, :], o[t*k + j, :]>: the gradient of mi_moe_combine w.r.t. the gates.  H % 8 == 0. */
+/* d_gates[t, j] = <dy[t, :], o[t*k + j, :]>: the gradient of mi_moe_combine w.r.t. the gates.  H % 8 == 0 (F32: H % 4 == 0). */
 int mi_moe_combine_grad_gates(const void* o, const void* dy, void* d_gates, int T, int k, int H, int dtype,
                               mi_moe_stream_t stream);
 

@@ -20,22 +20,24 @@ def _ops():
     return ops
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("L,I,k", [(1, 8, 1), (36, 64, 2), (512, 512, 8), (4098, 1408, 6)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("L,I,k", [(1, 8, 1), (36, 64, 2), (512, 512, 8), (4098, 1408, 6), (30, 12, 3)])
 @pytest.mark.parametrize("routed", [False, True])
 def test_swiglu_backward(device, dtype, L, I, k, routed):
     """d_h, g * a and the router-weight gradient against autograd through z = sum_i g_i <c_i, up_i * silu(gate_i)>
     (c = d_act plays the role of the upstream gradient w_proj^T dy)."""
+    if I % 8 and dtype != torch.float32:
+        pytest.skip("a row of 16-bit values must be whole 16-byte chunks")
     g = torch.Generator().manual_seed(L * 31 + I)
     h = (torch.randn(L, 2 * I, generator=g) * 2).to(dtype)
     d_act = torch.randn(L, I, generator=g).to(dtype)
     gates = torch.rand(L // k, k, generator=g).to(dtype) if routed else None
     ss = torch.randperm(L, generator=g).to(torch.int32) if routed else None
 
-    hf = h.float().requires_grad_(True)
+    hf = h.float().clone().requires_grad_(True)
     a = hf[:, :I] * F.silu(hf[:, I:])
     if routed:
-        gf = gates.float().requires_grad_(True)
+        gf = gates.float().clone().requires_grad_(True)
         g_rows = gf.reshape(-1)[ss.long()].unsqueeze(-1)
     else:
         g_rows = 1.0
@@ -45,7 +47,7 @@ def test_swiglu_backward(device, dtype, L, I, k, routed):
         h.to(device), d_act.to(device), None if gates is None else gates.to(device),
         None if ss is None else ss.to(device), want_act=True, want_gate_grad=routed)
     assert d_h.dtype == dtype and tuple(d_h.shape) == (L, 2 * I)
-    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2e-6}[dtype]
     torch.testing.assert_close(d_h.cpu().float(), hf.grad, rtol=2 * eps, atol=1e-6)
     torch.testing.assert_close(act_g.cpu().float(), (g_rows * a).detach(), rtol=2 * eps, atol=1e-6)
     if routed:
@@ -59,7 +61,7 @@ def test_swiglu_backward(device, dtype, L, I, k, routed):
 @pytest.mark.parametrize("L,I", [(1, 8), (77, 136), (1000, 512), (5, 100)])
 def test_swiglu_forward(device, dtype, L, I):
     """a = up * silu(gate) of a stored pre-activation against the closed form in fp64 on the same rounded h
-    (activations/glu.py:42-43); (5, 100) and fp32 take the torch form inside the wrapper."""
+    (activations/glu.py:42-43); (5, 100) in a 16-bit dtype takes the torch form inside the wrapper."""
     g = torch.Generator().manual_seed(L + I)
     h = (torch.randn(L, 2 * I, generator=g) * 2).to(dtype)
     got = _ops().swiglu_forward(h.to(device))
@@ -84,16 +86,18 @@ def test_swiglu_backward_empty_and_errors(device):
                             torch.zeros(4, 16, device=device, dtype=torch.bfloat16), want_gate_grad=True)
     from dolomite_engine_amd._lib import MiMoeError
 
-    with pytest.raises(MiMoeError):  # fp32 is not a dtype of this kernel
-        ops.swiglu_backward(torch.zeros(4, 32, device=device), torch.zeros(4, 16, device=device))
+    with pytest.raises(MiMoeError):  # fp32: I % 4 != 0
+        ops.swiglu_backward(torch.zeros(4, 12, device=device), torch.zeros(4, 6, device=device))
     with pytest.raises(MiMoeError):  # I % 8 != 0
         ops.swiglu_backward(torch.zeros(4, 24, device=device, dtype=torch.bfloat16),
                             torch.zeros(4, 12, device=device, dtype=torch.bfloat16))
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("T,k,H", [(1, 1, 8), (5, 2, 64), (300, 8, 1536), (64, 6, 4096), (1027, 2, 520)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,k,H", [(1, 1, 8), (5, 2, 64), (300, 8, 1536), (64, 6, 4096), (1027, 2, 520), (9, 3, 12)])
 def test_combine_grad_gates(device, dtype, T, k, H):
+    if H % 8 and dtype != torch.float32:
+        pytest.skip("a row of 16-bit values must be whole 16-byte chunks")
     g = torch.Generator().manual_seed(T + k + H)
     o = torch.randn(T * k, H, generator=g).to(dtype)
     dy = torch.randn(T, H, generator=g).to(dtype)
@@ -103,7 +107,7 @@ def test_combine_grad_gates(device, dtype, T, k, H):
 
     got = _ops().combine_grad_gates(o.to(device), dy.to(device), k)
     assert got.dtype == dtype and tuple(got.shape) == (T, k)
-    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2e-6}[dtype]
     # an fp32 dot product of H terms rounded once; the absolute term covers cancellation
     torch.testing.assert_close(got.cpu().float(), gates.grad, rtol=2 * eps, atol=1e-4 * H ** 0.5)
 
