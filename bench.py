@@ -248,10 +248,45 @@ def measure_ceilings(w, inputs, device, iters=20):
     ms3 = _time_ms(lambda: dst.copy_(src), 10)
     out["copy_1gib"] = {"ms": ms3, "gbs_read_plus_write": 2.0 * (1 << 30) / (ms3 * 1e-3) / 1e9,
                         "frac": 2.0 * (1 << 30) / (ms3 * 1e-3) / 1e9 / PEAK_HBM_GBS}
-    out["note"] = ("torch.mm (vendor dense bf16 GEMM) and Tensor.copy_ timed with HIP events in this process; "
-                   "frac is of the 2.5 PFLOP/s bf16 MFMA peak / the 8 TB/s HBM peak")
     del src, dst
+    out["gemm_inner_loop"] = measure_inner_loop_probes(device)
+    out["note"] = ("torch.mm (vendor dense bf16 GEMM) and Tensor.copy_ timed with HIP events in this process; "
+                   "gemm_inner_loop: the library's diagnostic kernels (mi_moe_probe_kloop) on random bf16 data; "
+                   "frac is of the 2.5 PFLOP/s bf16 MFMA peak / the 8 TB/s HBM peak")
     torch.cuda.empty_cache()
+    return out
+
+
+def measure_inner_loop_probes(device, slices=6144):
+    """The pieces of the persistent grouped GEMM's inner loop in isolation (mi_moe_probe_kloop: one workgroup per
+    CU, the GEMM's own 256 x 256 tile, slice, ring and schedule, on 2 MiB of L2-resident random bf16 data): the
+    matrix instructions alone, with the LDS fragment reads, the L2 -> LDS DMA alone, and all of it together.  What
+    "all of it" reaches is the ceiling of the GEMM's K loop on this GPU -- before gather, expert tails, tile
+    boundaries and epilogues."""
+    import torch
+
+    from dolomite_engine_amd import _lib
+
+    lib = _lib.load()
+    g = torch.Generator(device="cpu").manual_seed(7)
+    data = torch.randn((2 << 20) // 2 + 4096, generator=g).to(torch.bfloat16).to(device)
+    sink = torch.empty(lib.mi_moe_probe_sink_bytes(), dtype=torch.uint8, device=device)
+    cus = sink.numel() // (512 * 4)
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {"workgroups": cus, "slices_per_workgroup": slices}
+    for mode, name in ((0, "mfma_only"), (1, "mfma_plus_lds_reads"), (2, "dma_only"), (3, "all_pingpong")):
+        def launch():
+            _lib.check(lib.mi_moe_probe_kloop(mode, data.data_ptr(), data.numel() * 2, slices, sink.data_ptr(),
+                                              sink.numel(), stream))
+        ms = _time_ms(launch, 5, warmup=2)
+        rec = {"ms": ms}
+        if mode != 2:
+            tf = 2.0 * 256 * 256 * 32 * slices * cus / (ms * 1e-3) / 1e12
+            rec.update(tflops=tf, frac=tf / PEAK_BF16_TFLOPS)
+        if mode >= 2:
+            rec["l2_to_lds_tbs"] = 32768.0 * slices * cus / (ms * 1e-3) / 1e12
+        out[name] = rec
+    del data, sink
     return out
 
 

@@ -60,6 +60,8 @@ SIGNATURES: dict[str, tuple] = {
     "mi_moe_aux_loss_workspace_bytes": (_sz, [_i, _i]),
     "mi_moe_aux_loss": (_i, [_vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "mi_moe_aux_loss_backward": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "mi_moe_probe_sink_bytes": (_sz, []),
+    "mi_moe_probe_kloop": (_i, [_i, _vp, _sz, _i, _vp, _sz, _vp]),
     "mi_moe_fp8_tiled_bytes": (_sz, [_i, _i, _i, _i]),
     "mi_moe_up_swiglu_fp8": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "mi_moe_down_fp8": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),

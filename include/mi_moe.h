@@ -367,6 +367,22 @@ int mi_moe_down_fp8(const void* act, const void* w_proj_q, const float* w_proj_s
                     const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
                     int E, int dtype, int w_tiled, mi_moe_stream_t stream);
 
+/*
+ * Diagnostics (no counterpart in the reference; nothing in the layer calls them): the pieces of the persistent
+ * grouped GEMM's inner loop in isolation, for a benchmark that wants a measured ceiling beside the GEMM's own
+ * figure.  One workgroup of eight waves per compute unit runs `slices` K slices of a 256 x 256 bf16 tile the way
+ * the GEMM does (32 matrix instructions 16x16x32, twelve 16-byte LDS fragment reads and four 1 KiB DMA
+ * instructions per wave and slice, ring of four 32 KiB stages) with parts switched off:
+ *   mode 0  matrix instructions only        mode 1  + the LDS fragment reads
+ *   mode 2  DMA only (L2 -> LDS fill)       mode 3  everything, in the GEMM's two-group ping-pong schedule
+ * Per workgroup and slice: 2 * 256 * 256 * 32 flops, 32 KiB of DMA.  data: at least 2 MiB + 4 KiB of bytes of the
+ * caller's choice (random bf16 values draw more power than zeros), 16-byte aligned, read only; sink:
+ * mi_moe_probe_sink_bytes() bytes that the kernels write (one float per thread, so that nothing is optimised away).
+ */
+size_t mi_moe_probe_sink_bytes(void);
+int mi_moe_probe_kloop(int mode, const void* data, size_t data_bytes, int slices, void* sink, size_t sink_bytes,
+                       mi_moe_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

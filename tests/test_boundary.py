@@ -100,7 +100,13 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_sort_bin_static(ctypes.c_void_p(256), 1 << 20, 8, 1000, ctypes.c_void_p(256), ctypes.c_void_p(256),
                                       ctypes.c_void_p(256), None) == -7
     assert lib.mi_moe_swiglu_forward(None, None, 4, 12, _lib.BF16, None) == E_UNSUP
-    assert lib.mi_moe_swiglu_forward(None, None, 4, 16, _lib.F32, None) == E_DTYPE
+    assert lib.mi_moe_swiglu_forward(None, None, 4, 16, 7, None) == E_DTYPE
+    assert lib.mi_moe_swiglu_forward(None, None, 4, 6, _lib.F32, None) == E_UNSUP   # fp32 rows: whole 16-byte chunks too
+    assert lib.mi_moe_swiglu_forward(None, None, 4, 12, _lib.F32, None) == E_NULL
+    # the diagnostic loop probes validate like everything else
+    assert lib.mi_moe_probe_kloop(4, None, 4 << 20, 10, None, 0, None) == E_SHAPE
+    assert lib.mi_moe_probe_kloop(0, None, 1 << 20, 10, None, 0, None) == E_SHAPE
+    assert lib.mi_moe_probe_kloop(0, None, 4 << 20, 10, None, 0, None) == E_NULL
     assert lib.mi_moe_swiglu_forward(None, None, 4, 16, _lib.BF16, None) == E_NULL
     assert lib.mi_moe_swiglu_forward(None, None, 0, 16, _lib.BF16, None) == 0
     assert lib.mi_moe_grouped_wgrad_naive(None, None, None, None, None, None, 16, 8, 8, 4, 7, None) == E_DTYPE
@@ -140,7 +146,7 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_grouped_wgrad(None, None, None, None, None, None, None, 0, 16, 16, 16, 8, 8, 4, _lib.BF16, None) == E_NULL
     assert lib.mi_moe_grouped_wgrad_workspace_bytes(262144, 40, 1024, 1536) > 0
     assert lib.mi_moe_swiglu_backward(None, None, None, None, None, None, None, 4, 12, _lib.BF16, None) == E_UNSUP
-    assert lib.mi_moe_swiglu_backward(None, None, None, None, None, None, None, 4, 16, _lib.F32, None) == E_DTYPE
+    assert lib.mi_moe_swiglu_backward(None, None, None, None, None, None, None, 4, 16, 7, None) == E_DTYPE
     assert lib.mi_moe_swiglu_backward(None, None, None, None, None, None, None, 0, 16, _lib.BF16, None) == 0
     assert lib.mi_moe_combine_grad_gates(None, None, None, 4, 2, 16, _lib.BF16, None) == E_NULL
     assert lib.mi_moe_aux_loss(None, None, None, None, 0, 4, 300, 2, _lib.BF16, None) == E_UNSUP

@@ -560,3 +560,30 @@ def test_fp8_random_shapes(device, seed):
                                ("down row-major", o_r, ref_o)):
             err = (got.cpu().float() - ref).abs().max().item()
             assert err <= 2e-2 * ref.abs().max().item() + 2e-3, (case, name, err)
+
+
+def test_inner_loop_probes_run(device):
+    """The diagnostic kernels behind bench.py's `ceilings.gemm_inner_loop` (mi_moe_probe_kloop): every mode runs to
+    completion on a short loop, writes its whole sink, and the matrix modes agree with each other -- modes 0, 1 and 3
+    multiply the same first ring contents when the data repeats every 64 bytes of K."""
+    from dolomite_engine_amd import _lib
+
+    lib = _lib.load()
+    n = (2 << 20) // 2 + 4096
+    data = torch.full((n,), 0.5, dtype=torch.bfloat16, device=device)   # constant data: every slice is the same
+    sink_bytes = lib.mi_moe_probe_sink_bytes()
+    assert sink_bytes > 0 and sink_bytes % (512 * 4) == 0
+    stream = torch.cuda.current_stream().cuda_stream
+    sums = {}
+    for mode in (0, 1, 2, 3):
+        sink = torch.full((sink_bytes // 4,), float("nan"), dtype=torch.float32, device=device)
+        print(f"probe mode {mode}", flush=True)
+        rc = lib.mi_moe_probe_kloop(mode, data.data_ptr(), n * 2, 64, sink.data_ptr(), sink_bytes, stream)
+        assert rc == 0, lib.mi_moe_strerror(rc).decode()
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(sink).all())
+        sums[mode] = sink.clone()
+    # 64 slices x 32 k of 0.5 * 0.5 per output element, 128 elements summed per thread
+    want = 64 * 32 * 0.25 * 128
+    for mode in (0, 1, 3):
+        assert bool((sums[mode] == want).all()), mode
