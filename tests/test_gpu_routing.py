@@ -311,3 +311,58 @@ def test_router_fused_sort_limits(device):
     assert not ops.router_fused_sort_supported(torch.zeros(2048, 4096, dtype=torch.bfloat16, device=device), 64, 2)  # gate weights beyond LDS
     assert not ops.router_fused_sort_supported(x[:1024], 64, 9)  # k beyond the fused router
     assert ops.router_fused_sort_supported(x[:1024], 64, 8)      # 8192 slots: the one-block sort's limit
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_routing_random_shapes(device, seed):
+    """Random shapes through every form of the routing stage -- streaming router, general router (fp32, many
+    experts, large k), router + sort in both its forms, stand-alone sort -- against the oracle: routing bit-exact on
+    the device's own logits, sort bit-exact, and the fused forms bit-identical to the separate calls."""
+    import random
+
+    ops = _ops()
+    rnd = random.Random(seed)
+    for case in range(24):
+        dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+        E = rnd.choice([1, 2, 5, 8, 16, 40, 64, 65, 100, 128, 200, 256])
+        k = min(rnd.choice([1, 2, 3, 6, 8, 9, 20]), E)
+        T = rnd.choice([1, 3, 16, 17, 100, 512, 1024, 1025, 1500, 4099, 9000])
+        H = 16 * rnd.choice([1, 2, 3, 8, 17, 48, 64, 96])
+        bias = rnd.choice([False, True])
+        g = torch.Generator().manual_seed(seed * 7919 + case)
+        x = torch.randn(T, H, generator=g).to(dtype)
+        w = (torch.randn(E, H, generator=g) * 0.05).to(dtype)
+        b = (torch.randn(E, generator=g) * 0.3) if bias else None
+        print(f"routing random seed {seed} case {case}: T={T} H={H} E={E} k={k} {dtype} bias={bias}", flush=True)
+        xd, wd, bd = x.to(device), w.to(device), None if b is None else b.to(device)
+        assert ops.router_fused_supported(xd, E, k)
+        logits, gates, idx = ops.router_fused(xd, wd, k, bias=bd, return_logits=True)
+        ref_logits = oracle.router_logits(x, w, b)
+        tol = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.bfloat16: dict(rtol=1.6e-2, atol=2e-3),
+               torch.float16: dict(rtol=2e-3, atol=1e-3)}[dtype]
+        torch.testing.assert_close(logits.cpu().float(), ref_logits.float(), **tol)
+        vals, ref_idx = oracle.topk_canonical(logits.cpu(), k)
+        assert torch.equal(idx.cpu().long(), ref_idx), case
+        ref_gates = oracle.softmax_topk(vals, dtype)
+        if dtype == torch.float32:
+            torch.testing.assert_close(gates.cpu(), ref_gates, rtol=1e-5, atol=1e-7)
+        else:
+            assert (gates.cpu().view(torch.int16).int() - ref_gates.view(torch.int16).int()).abs().max() <= 1
+        se, ss, off = ops.sort_bin(idx, E)
+        ose, oss, ooff = oracle.sort_bin(ref_idx, E)
+        assert torch.equal(se.cpu().long(), ose) and torch.equal(ss.cpu().long(), oss) and torch.equal(off.cpu().long(), ooff)
+        if ops.router_fused_sort_supported(xd, E, k):
+            l2, g2, i2, se2, ss2, off2 = ops.router_fused_sort(xd, wd, k, bias=bd, return_logits=True)
+            assert torch.equal(l2, logits) and torch.equal(g2, gates) and torch.equal(i2, idx), case
+            assert torch.equal(se2, se) and torch.equal(ss2, ss) and torch.equal(off2, off), case
+        # backward of the routing: d logits for random incoming gradients against autograd
+        d_gates = torch.randn(T, k, generator=g).to(dtype)
+        got = ops.router_dlogits(logits, idx, d_gates.to(device), None).cpu()
+        lg = logits.cpu().clone().requires_grad_(True)
+        (torch.softmax(lg.gather(-1, ref_idx).float(), dim=-1).to(dtype) * d_gates).sum().backward()
+        if dtype == torch.float32:
+            torch.testing.assert_close(got, lg.grad, rtol=1e-4, atol=1e-6)
+        else:
+            steps = (got.view(torch.int16).int() - lg.grad.view(torch.int16).int()).abs()
+            close = (got.float() - lg.grad.float()).abs() <= 1e-3 * lg.grad.float().abs() + 2e-6
+            assert bool(((steps <= 1) | close).all()), case
