@@ -17,6 +17,10 @@
 //   * An expert's rows are cut into groups of `chunk` rows; a work item is one 256 x 256 output tile of one
 //     group.  Items are dealt so that the 32 workgroups of an XCD work on the tiles of the same few groups at
 //     the same time: the group's rows are then fetched from HBM once per XCD and shared through its L2.
+//     Which XCD takes which groups is planned by a one-workgroup kernel in front: the groups are ranked by size,
+//     longest first, and dealt to the eight XCDs back and forth (0..7, 7..0, ...), so that the XCDs get equal
+//     work up to a small group and every XCD ends on its shortest items.  (Dealing the sorted rows into eight
+//     equal ranges instead leaves the XCDs up to one group apart and costs 10 - 20 % under skewed loads.)
 //     An item of an expert with several groups writes an fp32 partial tile and a second kernel sums the partials
 //     of the expert in group order and rounds once (deterministic); an expert with one group is written directly,
 //     one without rows gets zeros from the second kernel.
@@ -53,7 +57,8 @@ struct WgradArgs {
   const int32_t* expert_offsets;  // (E,) inclusive ends of the experts' row ranges
   float* partial;                 // [group][M][N]
   void* dw;                       // (E, M, N): written directly for an expert with a single group
-  int* next_item;                 // [8] per-XCD work counters, zero on entry
+  int* next_item;                 // plan: [0..8) per-XCD work counters, zero on entry; [8..17) first slot of each XCD
+                                  // in the list; [32..) the groups in the order the XCDs work through them
   int L, M, N, E, chunk, m_tiles, n_tiles;
 };
 
@@ -130,38 +135,16 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
   const int wm = wave & 3, wn = wave >> 2;
 
   wgrad_build_table(a.expert_offsets, a.E, a.chunk, etab, lane, wave);
-  const int total_groups = etab[2 * (a.E - 1)];
   const int tiles = a.m_tiles * a.n_tiles;
   const int xcd = blockIdx.x & 7;
 
   // An expert with n rows has ceil(n / chunk) groups of equal size (a multiple of 32 rows, the last one shorter).
   auto group_rows = [&](int n, int groups) { return ((n + groups - 1) / groups + 31) & ~31; };
-  // first group that starts at or after sorted row `b` (wave-uniform)
-  auto group_at = [&](int b) -> int {
-    int res = total_groups;
-    for (int e0 = 0; e0 < a.E; e0 += 64) {
-      const int e = e0 + lane;
-      const int end = e < a.E ? etab[2 * e + 1] : 0x7fffffff;
-      const uint64_t hit = __ballot(end > b);
-      if (hit) {
-        const int ex = e0 + __ffsll((long long)hit) - 1;
-        if (ex < a.E) {
-          const int first = ex > 0 ? etab[2 * (ex - 1)] : 0;
-          const int prev = ex > 0 ? etab[2 * (ex - 1) + 1] : 0;
-          const int groups = etab[2 * ex] - first;
-          const int rows = group_rows(etab[2 * ex + 1] - prev, groups);
-          const int gi = (b - prev + rows - 1) / rows;
-          res = first + (gi < groups ? gi : groups);
-        }
-        break;
-      }
-    }
-    return __builtin_amdgcn_readfirstlane(res);
-  };
-  // every XCD takes the groups that start in its eighth of the sorted rows: equal work up to one group
-  const int gbeg = group_at((int)((long)a.L * xcd >> 3));
-  const int gend = xcd == 7 ? total_groups : group_at((int)((long)a.L * (xcd + 1) >> 3));
-  const int items_x = (gend - gbeg) * tiles;
+  // this XCD's groups: slots [xfirst, xfirst + xgroups) of the planned list
+  const int xfirst = a.next_item[8 + xcd];
+  const int xgroups = a.next_item[8 + xcd + 1] - xfirst;
+  const int* __restrict__ xlist = a.next_item + 32 + xfirst;
+  const int items_x = xgroups * tiles;
 
   // ---- loader role: waves 0-3 stage operand A, waves 4-7 operand B; each wave rows 8 wq .. 8 wq + 7 of a slice --
   const bool load_b = wave >= 4;
@@ -198,7 +181,7 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
     const int item = __builtin_amdgcn_readfirstlane(*item_slot);
     __syncthreads();
     if (item >= items_x) break;
-    const int grp = gbeg + item / tiles;
+    const int grp = __builtin_amdgcn_readfirstlane(xlist[item / tiles]);
     // A group's tiles are numbered in bands of 8 row tiles, column tile slowest inside a band: the 32 workgroups
     // of the XCD, which hold 32 consecutive items, then cover 8 x 4 tiles -- 12 operand slabs for 32 tiles.  (Row
     // tile fastest over all of them would re-read every A slab once per column tile: with 112 x 16 tiles that is
@@ -398,8 +381,68 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
   else run_items(std::false_type{});
 }
 
-__global__ void wgrad_zero_counters_kernel(int* counters) {
-  if (threadIdx.x < 8) counters[threadIdx.x] = 0;
+// Plan of one launch (one workgroup, in front of the main kernel): zero the eight work counters, rank the
+// groups by their number of rows (longest first, ties in row order) and deal them to the XCDs back and forth.
+//   plan[0..8)   work counters
+//   plan[8..17)  first slot of XCD x in the list (slot 8 + 8 = one past the end)
+//   plan[32..)   group numbers (row order numbering, as the partial slabs and the reduction use) by slot
+// Up to WGRAD_PLAN_SORT groups are ranked; beyond that the groups are dealt in row order.
+#define WGRAD_PLAN_SORT 8192
+__global__ __launch_bounds__(1024) void wgrad_plan_kernel(const int32_t* __restrict__ offsets, int E, int chunk,
+                                                          int* __restrict__ plan) {
+  __shared__ int first[WGRAD_MAX_E + 1];  // groups in front of expert e
+  __shared__ int rows[WGRAD_PLAN_SORT];
+  const int tid = threadIdx.x;
+  if (tid < 8) plan[tid] = 0;
+  if (tid == 0) {
+    int g = 0;
+    for (int e = 0; e < E; ++e) {
+      first[e] = g;
+      const int n = offsets[e] - (e > 0 ? offsets[e - 1] : 0);
+      g += (n + chunk - 1) / chunk;
+    }
+    first[E] = g;
+  }
+  __syncthreads();
+  const int G = first[E];
+  const bool sorted = G <= WGRAD_PLAN_SORT;
+  if (sorted) {
+    // rows of every group: group i of an expert with n rows in `groups` groups of `per` rows each
+    for (int e = tid; e < E; e += blockDim.x) {
+      const int n = offsets[e] - (e > 0 ? offsets[e - 1] : 0);
+      const int groups = first[e + 1] - first[e];
+      if (groups == 0) continue;
+      const int per = ((n + groups - 1) / groups + 31) & ~31;
+      for (int i = 0; i < groups; ++i) {
+        const int r1 = (i + 1) * per < n ? (i + 1) * per : n;
+        rows[first[e] + i] = r1 - i * per;
+      }
+    }
+  }
+  __syncthreads();
+  // XCD x gets the ranks 16 j + x and 16 j + 15 - x: G / 8 full rounds and part of one more
+  const int full = G >> 3, rem = G & 7;
+  if (tid < 9) {
+    int start = 0;
+    for (int x = 0; x < tid; ++x) start += full + (((full & 1) == 0 ? x < rem : x >= 8 - rem) ? 1 : 0);
+    plan[8 + tid] = start;
+  }
+  for (int g = tid; g < G; g += blockDim.x) {
+    int rank = g;
+    if (sorted) {
+      const int mine = rows[g];
+      rank = 0;
+      for (int o = 0; o < G; ++o) {
+        const int r = rows[o];
+        rank += (r > mine || (r == mine && o < g)) ? 1 : 0;
+      }
+    }
+    const int round = rank >> 3, pos = rank & 7;
+    const int x = (round & 1) == 0 ? pos : 7 - pos;
+    int start = 0;
+    for (int y = 0; y < x; ++y) start += full + (((full & 1) == 0 ? y < rem : y >= 8 - rem) ? 1 : 0);
+    plan[32 + start + round] = g;
+  }
 }
 
 // dW[e] = sum of expert e's partial slabs in group order, rounded once (experts with several groups); zeros for an
@@ -436,22 +479,29 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restri
   }
 }
 
-// rows per group: enough groups for about four items per CU, between 256 and 8192 rows, a multiple of 32
+// Rows per group: between 256 and 16384, a multiple of 32, and few enough groups that the fp32 partial tiles of
+// the experts with several groups stay cheap: about 384 items (1.5 per CU) before the cap.  Measured on the
+// Granite-3B-A800M shapes (262144 rows, 40 experts): every megabyte of partial tiles costs about as much as
+// 0.07 % of the products, so long groups beat groups of 3040 - 6080 rows (about four items per CU) by 4 - 7 %
+// under skewed loads and by 12 - 18 % under an even load (where no expert is split any more); the longest-first
+// plan keeps the few long items balanced.
 static int wgrad_chunk(int L, int M, int N) {
   const long tiles = (long)mi_ceil_div(M, 256) * mi_ceil_div(N, 256);
-  long groups = (1024 + tiles - 1) / tiles;
+  long groups = (384 + tiles - 1) / tiles;
   long chunk = L / (groups > 0 ? groups : 1);
-  if (chunk > 8192) chunk = 8192;
+  if (chunk > 16384) chunk = 16384;
   if (chunk < 256) chunk = 256;
   return (int)(chunk / 32 * 32);
 }
 
 static long wgrad_max_groups(int L, int E, int chunk) { return (long)L / chunk + (E < L ? E : L); }
+static size_t wgrad_plan_bytes(long groups) { return ((size_t)(32 + groups) * sizeof(int) + 255) / 256 * 256; }
 
 extern "C" size_t mi_moe_grouped_wgrad_workspace_bytes(int L, int E, int M, int N) {
   if (L < 1 || E < 1 || M < 1 || N < 1) return 0;
-  // [partial slabs][8 work counters, padded to 256 bytes]
-  return (size_t)wgrad_max_groups(L, E, wgrad_chunk(L, M, N)) * (size_t)M * (size_t)N * sizeof(float) + 256;
+  // [partial slabs][plan: 32 ints (work counters, first slots) + one int per group, padded to 256 bytes]
+  const long groups = wgrad_max_groups(L, E, wgrad_chunk(L, M, N));
+  return (size_t)groups * (size_t)M * (size_t)N * sizeof(float) + wgrad_plan_bytes(groups);
 }
 
 extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const void* b, const int32_t* b_idx,
@@ -480,7 +530,7 @@ extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const v
   if (L > 0) {
     g.next_item = reinterpret_cast<int*>(static_cast<unsigned char*>(workspace) +
                                          (size_t)wgrad_max_groups(L, E, g.chunk) * (size_t)M * (size_t)N * sizeof(float));
-    hipLaunchKernelGGL(wgrad_zero_counters_kernel, dim3(1), dim3(64), 0, s, g.next_item);
+    hipLaunchKernelGGL(wgrad_plan_kernel, dim3(1), dim3(1024), 0, s, expert_offsets, E, g.chunk, g.next_item);
   }
   g.m_tiles = mi_ceil_div(M, 256);
   g.n_tiles = mi_ceil_div(N, 256);
