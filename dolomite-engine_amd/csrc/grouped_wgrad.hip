@@ -391,14 +391,17 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
 __global__ __launch_bounds__(1024) void wgrad_plan_kernel(const int32_t* __restrict__ offsets, int E, int chunk,
                                                           int* __restrict__ plan) {
   __shared__ int first[WGRAD_MAX_E + 1];  // groups in front of expert e
+  __shared__ int ends[WGRAD_MAX_E];       // the offsets (one round trip to memory for all of them)
   __shared__ int rows[WGRAD_PLAN_SORT];
   const int tid = threadIdx.x;
   if (tid < 8) plan[tid] = 0;
+  for (int e = tid; e < E; e += blockDim.x) ends[e] = offsets[e];
+  __syncthreads();
   if (tid == 0) {
     int g = 0;
     for (int e = 0; e < E; ++e) {
       first[e] = g;
-      const int n = offsets[e] - (e > 0 ? offsets[e - 1] : 0);
+      const int n = ends[e] - (e > 0 ? ends[e - 1] : 0);
       g += (n + chunk - 1) / chunk;
     }
     first[E] = g;
@@ -409,7 +412,7 @@ __global__ __launch_bounds__(1024) void wgrad_plan_kernel(const int32_t* __restr
   if (sorted) {
     // rows of every group: group i of an expert with n rows in `groups` groups of `per` rows each
     for (int e = tid; e < E; e += blockDim.x) {
-      const int n = offsets[e] - (e > 0 ? offsets[e - 1] : 0);
+      const int n = ends[e] - (e > 0 ? ends[e - 1] : 0);
       const int groups = first[e + 1] - first[e];
       if (groups == 0) continue;
       const int per = ((n + groups - 1) / groups + 31) & ~31;
