@@ -89,6 +89,7 @@ struct GemmArgs {
   int N;        // output columns (SwiGLU: I, with 2N weight rows per expert)
   int E;
   int kdiv;     // gather divisor (top-k) for scattered inputs
+  int kshift;   // log2(kdiv) if kdiv is a power of two, else -1 (set by launch_persistent)
   int n_tiles;  // column tiles per row tile
   int gather;   // input row of sorted row i is sorted_scattered[i] / kdiv (else i)
   int scatter;  // output row of sorted row i is sorted_scattered[i] (else i)
@@ -938,7 +939,9 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
 #pragma unroll
     for (int j = 0; j < NLD; ++j) {
       if (j < NXLD) {
-        const int s = a.gather ? raw[j] / a.kdiv : raw[j];
+        // (top-k is a power of two in every configuration of the reference: a shift instead of a division per lane
+        // and tile; launch_persistent sets kshift to -1 otherwise)
+        const int s = !a.gather ? raw[j] : (a.kshift >= 0 ? raw[j] >> a.kshift : raw[j] / a.kdiv);
         ts.off[j] = ((uint32_t)s * (uint32_t)a.K + lchunk * 8) * (uint32_t)sizeof(T);
       } else if constexpr (WT) {
         // DMA instruction = two K rows of the slice; LDS piece lane % 32 of row krow holds the logical 16-byte
@@ -1038,12 +1041,16 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[nb][mb][i] = 0.f;
 
-  // eight instructions in a row share the activation operand
-  auto mfma_step = [&]() {
+  // eight instructions in a row share the activation operand.  The first slice of a tile multiplies onto a zero
+  // operand instead of the accumulators (an inline constant of the instruction), so that the accumulators need not
+  // be cleared between tiles: 128 moves per wave and tile, issued when the matrix pipe has nothing else to do.
+  auto mfma_step = [&](auto first_tag) {
+    constexpr bool FIRST = decltype(first_tag)::value;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mfma16<T>::run(wf[nb], xf[mb], acc[nb][mb]);
+      for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mfma16<T>::run(wf[nb], xf[mb], FIRST ? zero : acc[nb][mb]);
   };
 
   int g = 0;  // running K-slice count; slice g lives in ring stage g % NSTAGE
@@ -1054,7 +1061,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   // reading.  Every phase ends in a workgroup barrier; at each barrier one group has just issued its last MFMA
   // and the other has its operands in registers, so the matrix pipe of the SIMD never waits for LDS, DMA or the
   // barrier itself.
-  auto pp_slice = [&](const TileSrc& tcur, const TileSrc& tnext, bool from_next, int kload) {
+  auto pp_slice = [&](auto first_tag, const TileSrc& tcur, const TileSrc& tnext, bool from_next, int kload) {
     const int cur = g & (NSTAGE - 1), fill = (g + NSTAGE - 1) & (NSTAGE - 1);
     read_frags(cur);
     dma_slice(tcur, tnext, from_next, kload, fill);
@@ -1066,7 +1073,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     __builtin_amdgcn_sched_barrier(0);
     // (Signalling the second barrier a few matrix instructions early, so that they cover its release
     // latency, measured slower: the group's next memory phase then starts late and becomes the long one.)
-    mfma_step();
+    mfma_step(first_tag);
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -1085,15 +1092,32 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     int r[MP][32 / RPP];
   };
   auto load_out_rows = [&](const TileCoord& tc, OutRows& o) {
+    // (rows past the expert's end are never stored: with scattered output they read the index of its last row, so
+    // that the loads need no predicates)
+    const int row0 = tc.row_begin + wm * WTM + lane / EPI_CPR;
+    if (a.scatter) {
 #pragma unroll
-    for (int mp = 0; mp < MP; ++mp)
+      for (int mp = 0; mp < MP; ++mp)
 #pragma unroll
-      for (int it = 0; it < 32 / RPP; ++it) {
-        const int row = tc.row_begin + wm * WTM + mp * 32 + it * RPP + lane / EPI_CPR;
-        o.r[mp][it] = (a.scatter && row < tc.row_end) ? a.sorted_scattered[row] : row;
-      }
+        for (int it = 0; it < 32 / RPP; ++it) {
+          const int row = row0 + mp * 32 + it * RPP;
+          o.r[mp][it] = a.sorted_scattered[row < tc.row_end ? row : tc.row_end - 1];
+        }
+    } else {
+#pragma unroll
+      for (int mp = 0; mp < MP; ++mp)
+#pragma unroll
+        for (int it = 0; it < 32 / RPP; ++it) o.r[mp][it] = row0 + mp * 32 + it * RPP;
+    }
   };
-  auto epilogue = [&](const TileCoord& tc, const OutRows& orows) {
+  // INTERIOR: every row and column of the tile exists (all tiles but an expert's last row tile and a ragged last
+  // column tile), so the stores need no predicates; NT: non-temporal stores (see persistent_out_nt).  Both are
+  // compile-time forms of one body: the tile boundary is bound by instruction issue (no matrix work covers it),
+  // and a predicate, an exec-mask save / restore and a branch on the store's cache policy around each of a wave's
+  // 16 stores were a sixth of its instructions.
+  auto epilogue_as = [&](auto interior_tag, auto nt_tag, const TileCoord& tc, const OutRows& orows) {
+    constexpr bool INTERIOR = decltype(interior_tag)::value;
+    constexpr bool NT = decltype(nt_tag)::value;
     // the ring stage consumed last is free until the next tile's first memory phase refills it (the tile loop
     // puts a barrier between this epilogue and that refill)
     unsigned char* scratch = smem_raw + ((g + NSTAGE - 1) & (NSTAGE - 1)) * STAGE_BYTES + wave * EPI_BYTES;
@@ -1134,30 +1158,48 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
         // read back: lane -> row it*RPP + lane/EPI_CPR, 16-byte chunk lane%EPI_CPR
         const int cchunk = lane % EPI_CPR;
         const int col = tc.nt * BN + (GLU ? wn * (WTN / 2) : wn * WTN) + og * EPI_COLS + cchunk * 8;
+        // two reads at a time in front of their stores (one LDS latency for both): left alone, the compiler sinks
+        // each read into its store's predicated region and waits for it there; all four at once do not fit next
+        // to the accumulators
+        constexpr int RB = 2;
+        static_assert((32 / RPP) % RB == 0, "read-back batches");
 #pragma unroll
-        for (int it = 0; it < 32 / RPP; ++it) {
-          const int r = it * RPP + lane / EPI_CPR;
-          const u32x4 val = *reinterpret_cast<const u32x4*>(scratch + r * (EPI_COLS * 2) + ((cchunk ^ swz(r)) * 16));
-          const int row = tc.row_begin + wm * WTM + mp * 32 + r;
-          if (row < tc.row_end && col < a.N) {
-            u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)orow_of[mp][it] * a.N + col);
-            if (a.out_nt) {  // see persistent_out_nt
-              asm volatile("" ::: "memory");  // (the fences keep the compiler from merging the two stores into
-              __builtin_nontemporal_store(val, dst);  //  one plain store, hoisted or sunk out of the branch)
-              asm volatile("" ::: "memory");
-            } else {
-              *dst = val;
+        for (int it0 = 0; it0 < 32 / RPP; it0 += RB) {
+          __builtin_amdgcn_sched_barrier(0);  // (one batch's addresses and values live at a time)
+          u32x4 vals[RB];
+#pragma unroll
+          for (int j = 0; j < RB; ++j) {
+            const int r = (it0 + j) * RPP + lane / EPI_CPR;
+            vals[j] = *reinterpret_cast<const u32x4*>(scratch + r * (EPI_COLS * 2) + ((cchunk ^ swz(r)) * 16));
+          }
+#pragma unroll
+          for (int j = 0; j < RB; ++j) asm volatile("" : "+v"(vals[j]));
+#pragma unroll
+          for (int j = 0; j < RB; ++j) {
+            const int it = it0 + j;
+            const int r = it * RPP + lane / EPI_CPR;
+            const int row = tc.row_begin + wm * WTM + mp * 32 + r;
+            if (INTERIOR || (row < tc.row_end && col < a.N)) {
+              int orow = orow_of[mp][it];
+              asm volatile("" : "+v"(orow));  // (the address is formed here, not once per row and kept in registers)
+              u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)orow * a.N + col);
+              if constexpr (NT) __builtin_nontemporal_store(vals[j], dst);
+              else *dst = vals[j];
             }
           }
         }
       }
     }
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[nb][mb][i] = 0.f;
+  };
+  auto epilogue = [&](const TileCoord& tc, const OutRows& orows) {
+    const bool interior = tc.row_begin + BM <= tc.row_end && (tc.nt + 1) * BN <= a.N;
+    if (interior) {
+      if (a.out_nt) epilogue_as(std::true_type{}, std::true_type{}, tc, orows);
+      else epilogue_as(std::true_type{}, std::false_type{}, tc, orows);
+    } else {
+      if (a.out_nt) epilogue_as(std::false_type{}, std::true_type{}, tc, orows);
+      else epilogue_as(std::false_type{}, std::false_type{}, tc, orows);
+    }
   };
 
   // ---- a part of a split tile: accumulators -> workspace (one partial tile per (XCD, slot), fp32) -----------------
@@ -1208,9 +1250,12 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     // the ring runs on into the next tile: the last AHEAD slices refill with its first AHEAD.
     // group wn == 1 runs one phase behind group wn == 0 inside a tile; both leave the tile together
     if (wn == 1) __builtin_amdgcn_s_barrier();
-    for (int kt = 0; kt < nk_cur; ++kt) {
+    // (a tile or a part of one has at least NSTAGE slices: the first is never among the last AHEAD)
+    pp_slice(std::true_type{}, src_cur, src_next, false, k0_cur + AHEAD);
+    for (int kt = 1; kt < nk_cur; ++kt) {
       const bool from_next = kt >= nk_cur - AHEAD;
-      pp_slice(src_cur, src_next, from_next, from_next ? k0_next + kt + AHEAD - nk_cur : k0_cur + kt + AHEAD);
+      pp_slice(std::false_type{}, src_cur, src_next, from_next,
+               from_next ? k0_next + kt + AHEAD - nk_cur : k0_cur + kt + AHEAD);
     }
     if (wn == 0) __builtin_amdgcn_s_barrier();
     if (nk_cur != nk) {
@@ -1410,6 +1455,9 @@ static int launch_persistent(GemmArgs a, hipStream_t s) {
   int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok);
   if (rc != MI_MOE_OK) return rc;
   a.n_tiles = mi_ceil_div(a.N, BN);
+  a.kshift = -1;
+  if (a.kdiv > 0 && (a.kdiv & (a.kdiv - 1)) == 0)
+    for (a.kshift = 0; (1 << a.kshift) < a.kdiv;) ++a.kshift;
   if (!(a.remap & PERSIST_REMAP_FIXED) && a.n_tiles >= 8) a.remap |= PERSIST_REMAP_INTERLEAVE;  // (see there)
   int cus = 0;
   if ((rc = mi_cu_count(&cus)) != MI_MOE_OK) return rc;
