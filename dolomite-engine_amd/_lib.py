@@ -49,6 +49,7 @@ SIGNATURES: dict[str, tuple] = {
     "mi_moe_scattered_gemm_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "mi_moe_scattered_gemm_wt_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "mi_moe_up_swiglu_ws": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "mi_moe_up_swiglu_keep": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "mi_moe_combine": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mi_moe_combine_block_tail": (_i, [_vp, _vp, _vp, _vp, ctypes.c_float, _i, _vp, _i, _i, _i, _i, _vp]),
     "mi_moe_swiglu_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),

@@ -9,8 +9,9 @@ gradients (fp32 and odd shapes run a one-thread-per-element form of it; nothing 
 gradient, built on this package's forward kernels.
 
 Memory kept for the backward: x, the gates, the routing indices and -- by default -- the (L, 2I) pre-activation
-h of the up-projection (the forward then runs the up-projection unfused: grouped GEMM, then the element-wise
-SwiGLU on the stored h, as the reference does, moe.py:273-281); with ``keep_preactivation=False`` h is recomputed
+h of the up-projection (the up-projection then writes h next to the activation and forms the activation from
+the rounded h, as the reference's grouped GEMM followed by GLUActivation does, moe.py:273-281; shapes the tile
+kernel does not take run exactly those two steps); with ``keep_preactivation=False`` h is recomputed
 in the backward from x and the forward keeps its fused up-projection (one more grouped GEMM per step, L * 2I
 elements less memory).  The (L, I) activation follows from h, and the (L, H) expert outputs are never needed (the
 gradient of a router weight, <dy[t], w_proj[e] a>, is taken as <w_proj[e]^T dy[t], a>).
@@ -33,8 +34,7 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
     def forward(ctx, x, w_fc, w_proj, gates, sorted_scattered, expert_offsets, k, keep_preactivation=True):
         h = None
         if keep_preactivation:
-            h = ops.scattered_gemm(x, w_fc, k, sorted_scattered, expert_offsets, False, True)
-            act = ops.swiglu_forward(h)
+            act, h = ops.up_swiglu_keep(x, w_fc, k, sorted_scattered, expert_offsets)
         else:
             act = ops.up_swiglu(x, w_fc, k, sorted_scattered, expert_offsets)
         o = ops.scattered_gemm(act, w_proj, 1, sorted_scattered, expert_offsets, True, False)

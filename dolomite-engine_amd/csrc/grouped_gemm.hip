@@ -95,6 +95,7 @@ struct GemmArgs {
   int scatter;  // output row of sorted row i is sorted_scattered[i] (else i)
   int remap;    // XCD-aware tile order
   void* ws;     // persistent kernel: workspace for splitting the last round of tiles along K (or null)
+  void* pre;    // persistent SwiGLU kernel: (L, 2N) pre-activation output next to the activation (or null)
   int out_nt;   // persistent kernel: store the output non-temporal (set in run_gemm)
 };
 
@@ -837,8 +838,10 @@ __device__ __forceinline__ void persist_locate(const int* etab, int E, int n_til
   tc.expert = 0; tc.nt = 0; tc.row_begin = 0; tc.row_end = 1;  // unreachable for a valid tile id
 }
 
-template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool WT = false>
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool WT = false, bool KEEP_PRE = false>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(GemmArgs a) {
+  // KEEP_PRE: the SwiGLU form that also writes the pre-activation (a.pre), for training
+  static_assert(!KEEP_PRE || GLU, "the pre-activation belongs to the SwiGLU form");
   // WT: the expert weights are (K, N) row-major ("x @ W" with W as stored, the form both data gradients of the
   // backward take).  A K slice of them is 32 rows of 512 bytes; it is staged as it lies in HBM and the fragments
   // are read with the transposing LDS read (see read_frags).
@@ -1115,9 +1118,19 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   // compile-time forms of one body: the tile boundary is bound by instruction issue (no matrix work covers it),
   // and a predicate, an exec-mask save / restore and a branch on the store's cache policy around each of a wave's
   // 16 stores were a sixth of its instructions.
-  auto epilogue_as = [&](auto interior_tag, auto nt_tag, const TileCoord& tc, const OutRows& orows) {
+  // WHAT: 0 the kernel's result (with SwiGLU: up * silu(gate)); 1 / 2 (SwiGLU kernel keeping the pre-activation):
+  // the up / the gate half of h, into a.pre.  KEEP: the result is formed from the ROUNDED halves, as the separate
+  // activation kernel forms it from the stored h (swiglu_forward_kernel).
+  auto epilogue_as = [&](auto what_tag, auto interior_tag, auto nt_tag, auto keep_tag, const TileCoord& tc,
+                         const OutRows& orows) {
+    constexpr int WHAT = decltype(what_tag)::value;
     constexpr bool INTERIOR = decltype(interior_tag)::value;
     constexpr bool NT = decltype(nt_tag)::value;
+    constexpr bool KEEP = decltype(keep_tag)::value;
+    constexpr int OBX = WHAT == 0 ? OB : NB / 2;  // output column blocks of this form
+    static_assert(OBX % EPI_NB == 0, "epilogue pass shape");
+    T* __restrict__ dst_base = WHAT == 0 ? out : static_cast<T*>(a.pre);
+    const int ld = WHAT == 0 ? a.N : 2 * a.N;
     // the ring stage consumed last is free until the next tile's first memory phase refills it (the tile loop
     // puts a barrier between this epilogue and that refill)
     unsigned char* scratch = smem_raw + ((g + NSTAGE - 1) & (NSTAGE - 1)) * STAGE_BYTES + wave * EPI_BYTES;
@@ -1128,7 +1141,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
 #pragma unroll
     for (int mp = 0; mp < MP; ++mp) {
 #pragma unroll
-      for (int og = 0; og < OB / EPI_NB; ++og) {
+      for (int og = 0; og < OBX / EPI_NB; ++og) {
         // write the 32 x EPI_COLS block: a lane holds, per accumulator block, token row frow and the four
         // output columns 4 * fhalf + [0, 4)
 #pragma unroll
@@ -1141,9 +1154,17 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
             float v[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              if (GLU) {
-                const float up = acc[nb][mb][i];
-                const float gt = acc[nb + NB / 2][mb][i];
+              if (WHAT == 1) {
+                v[i] = acc[nb][mb][i];
+              } else if (WHAT == 2) {
+                v[i] = acc[nb + NB / 2][mb][i];
+              } else if (GLU) {
+                float up = acc[nb][mb][i];
+                float gt = acc[nb + NB / 2][mb][i];
+                if (KEEP) {
+                  up = Elt<T>::round(up);
+                  gt = Elt<T>::round(gt);
+                }
                 v[i] = up * gt * __builtin_amdgcn_rcpf(1.0f + __expf(-gt));
               } else {
                 v[i] = acc[nb][mb][i];
@@ -1157,7 +1178,9 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
         }
         // read back: lane -> row it*RPP + lane/EPI_CPR, 16-byte chunk lane%EPI_CPR
         const int cchunk = lane % EPI_CPR;
+        // column of the result (the predicate's), and of what this form writes
         const int col = tc.nt * BN + (GLU ? wn * (WTN / 2) : wn * WTN) + og * EPI_COLS + cchunk * 8;
+        const int dcol = WHAT == 2 ? a.N + col : col;
         // two reads at a time in front of their stores (one LDS latency for both): left alone, the compiler sinks
         // each read into its store's predicated region and waits for it there; all four at once do not fit next
         // to the accumulators
@@ -1182,7 +1205,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
             if (INTERIOR || (row < tc.row_end && col < a.N)) {
               int orow = orow_of[mp][it];
               asm volatile("" : "+v"(orow));  // (the address is formed here, not once per row and kept in registers)
-              u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)orow * a.N + col);
+              u32x4* dst = reinterpret_cast<u32x4*>(dst_base + (size_t)orow * ld + dcol);
               if constexpr (NT) __builtin_nontemporal_store(vals[j], dst);
               else *dst = vals[j];
             }
@@ -1191,14 +1214,32 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
       }
     }
   };
+  typedef std::integral_constant<int, 0> what_result;
+  typedef std::integral_constant<int, 1> what_up;
+  typedef std::integral_constant<int, 2> what_gate;
   auto epilogue = [&](const TileCoord& tc, const OutRows& orows) {
     const bool interior = tc.row_begin + BM <= tc.row_end && (tc.nt + 1) * BN <= a.N;
+    if constexpr (KEEP_PRE) {
+      {
+        // the activation and both halves of the pre-activation (plain stores: the backward reads them again)
+        if (interior) {
+          epilogue_as(what_result{}, std::true_type{}, std::false_type{}, std::true_type{}, tc, orows);
+          epilogue_as(what_up{}, std::true_type{}, std::false_type{}, std::true_type{}, tc, orows);
+          epilogue_as(what_gate{}, std::true_type{}, std::false_type{}, std::true_type{}, tc, orows);
+        } else {
+          epilogue_as(what_result{}, std::false_type{}, std::false_type{}, std::true_type{}, tc, orows);
+          epilogue_as(what_up{}, std::false_type{}, std::false_type{}, std::true_type{}, tc, orows);
+          epilogue_as(what_gate{}, std::false_type{}, std::false_type{}, std::true_type{}, tc, orows);
+        }
+        return;
+      }
+    }
     if (interior) {
-      if (a.out_nt) epilogue_as(std::true_type{}, std::true_type{}, tc, orows);
-      else epilogue_as(std::true_type{}, std::false_type{}, tc, orows);
+      if (a.out_nt) epilogue_as(what_result{}, std::true_type{}, std::true_type{}, std::false_type{}, tc, orows);
+      else epilogue_as(what_result{}, std::true_type{}, std::false_type{}, std::false_type{}, tc, orows);
     } else {
-      if (a.out_nt) epilogue_as(std::false_type{}, std::true_type{}, tc, orows);
-      else epilogue_as(std::false_type{}, std::false_type{}, tc, orows);
+      if (a.out_nt) epilogue_as(what_result{}, std::false_type{}, std::true_type{}, std::false_type{}, tc, orows);
+      else epilogue_as(what_result{}, std::false_type{}, std::false_type{}, std::false_type{}, tc, orows);
     }
   };
 
@@ -1444,13 +1485,13 @@ static int launch_dma(GemmArgs a, hipStream_t s) {
   return mi_launch_status();
 }
 
-template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool WT = false>
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool WT = false, bool KEEP_PRE = false>
 static int launch_persistent(GemmArgs a, hipStream_t s) {
   constexpr int BN = GLU ? BNW / 2 : BNW;
   constexpr int NW = WM * WN;
   static_assert(BM * BNW * 4 == PERSIST_WS_TILE_BYTES, "size of a partial tile in the workspace");
   const size_t lds = 4ull * (BM + BNW) * 32 * sizeof(T) + (size_t)a.E * 8;
-  auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, WT>;
+  auto kern = grouped_gemm_persistent_kernel<T, BM, BNW, WM, WN, GLU, WT, KEEP_PRE>;
   static std::atomic<uint64_t> lds_ok{0};  // the expert table makes lds vary with E: opt in to the most it can be
   int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok);
   if (rc != MI_MOE_OK) return rc;
@@ -1465,7 +1506,7 @@ static int launch_persistent(GemmArgs a, hipStream_t s) {
   long grid = cus < max_tiles ? cus : max_tiles;
   grid = (grid + 7) / 8 * 8;
   // no contraction length that a split could shorten by PERSIST_SPLIT_MIN_SAVED slices, or one slot per XCD
-  if (!persistent_may_split(a.K) || grid < 16) a.ws = nullptr;
+  if (!persistent_may_split(a.K) || grid < 16 || a.pre != nullptr) a.ws = nullptr;  // (the finishing launch writes the result only)
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, a);
   if ((rc = mi_launch_status()) != MI_MOE_OK || a.ws == nullptr) return rc;
   // the tiles that were cut: at most half of the slots of a round that was split hold tiles (rounded up: an odd
@@ -1623,7 +1664,7 @@ extern "C" int mi_moe_scattered_gemm_ws(const void* in, const void* w, void* out
   a.in = in; a.w = w; a.out = out;
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = K; a.N = N; a.E = E; a.kdiv = k; a.n_tiles = 0;
-  a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1; a.ws = ws;
+  a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1; a.ws = ws; a.pre = nullptr;
   return run_gemm(a, dtype, false, cfg, L, static_cast<hipStream_t>(stream));
 }
 
@@ -1649,7 +1690,7 @@ extern "C" int mi_moe_scattered_gemm_wt_ws(const void* in, const void* w_kn, voi
   a.in = in; a.w = w_kn; a.out = out;
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = K; a.N = N; a.E = E; a.kdiv = k; a.n_tiles = 0;
-  a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1; a.ws = ws;
+  a.gather = !grouped_in; a.scatter = !grouped_out; a.remap = 1; a.ws = ws; a.pre = nullptr;
   a.out_nt = persistent_out_nt(a, false, 2);
   if (!tiled_shape_ok(a, L, false, 2) || !persistent_ok(a)) return MI_MOE_EUNSUPPORTED;
   if (!tiled_aligned(a, 2)) return MI_MOE_EALIGN;
@@ -1682,8 +1723,33 @@ extern "C" int mi_moe_up_swiglu_ws(const void* x, const void* w_fc, void* act_ou
   a.in = x; a.w = w_fc; a.out = act_out;
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = H; a.N = I; a.E = E; a.kdiv = k; a.n_tiles = 0;
-  a.gather = 1; a.scatter = 0; a.remap = 1; a.ws = ws;
+  a.gather = 1; a.scatter = 0; a.remap = 1; a.ws = ws; a.pre = nullptr;
   return run_gemm(a, dtype, true, cfg, L, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mi_moe_up_swiglu_keep(const void* x, const void* w_fc, void* act_out, void* pre_out,
+                                     const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int H, int I,
+                                     int E, int k, int dtype, mi_moe_stream_t stream) {
+  int rc = check_common(x, w_fc, act_out, sorted_scattered, expert_offsets, L, H, I, E, k, dtype, true);
+  if (rc != MI_MOE_OK) return rc;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (L == 0) return MI_MOE_OK;
+  if (!pre_out) return MI_MOE_ENULL;
+  if (!mi_aligned(pre_out, 16)) return MI_MOE_EALIGN;
+  GemmArgs a;
+  a.in = x; a.w = w_fc; a.out = act_out;
+  a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
+  a.L = L; a.K = H; a.N = I; a.E = E; a.kdiv = k; a.n_tiles = 0;
+  a.gather = 1; a.scatter = 0; a.remap = 1; a.ws = nullptr; a.pre = pre_out;
+  // only the persistent kernel writes the pre-activation: shapes it does not take, and loads for which another
+  // kernel would be picked, are the caller's two-call path
+  if (!persistent_ok(a) || pick_cfg(a) != 7) return MI_MOE_EUNSUPPORTED;
+  if (!tiled_shape_ok(a, L, true, 2)) return MI_MOE_EUNSUPPORTED;
+  if (!tiled_aligned(a, 2)) return MI_MOE_EALIGN;
+  a.out_nt = 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MI_MOE_BF16) return launch_persistent<bf16_t, 256, 256, 4, 2, true, false, true>(a, s);
+  return launch_persistent<f16_t, 256, 256, 4, 2, true, false, true>(a, s);
 }
 
 extern "C" int mi_moe_up_swiglu_cfg(const void* x, const void* w_fc, void* act_out, const int32_t* sorted_scattered,

@@ -686,6 +686,38 @@ def up_swiglu(x: torch.Tensor, w_fc: torch.Tensor, k: int, sorted_scattered_idxs
     return act
 
 
+def up_swiglu_keep(x: torch.Tensor, w_fc: torch.Tensor, k: int, sorted_scattered_idxs: torch.Tensor,
+                   expert_offsets: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Up-projection for training: (act (L, I), h (L, 2I)) -- the activation and the pre-activation the backward
+    needs.  One launch (mi_moe_up_swiglu_keep) where the persistent tile kernel takes the problem, else the grouped
+    GEMM followed by the element-wise SwiGLU on the stored h; either way act is formed from the rounded h."""
+    _dev(x, w_fc, sorted_scattered_idxs, expert_offsets)
+    _no_grad(x, w_fc)
+    x = x.contiguous()
+    w_fc = w_fc.contiguous()
+    ss = _i32(sorted_scattered_idxs).contiguous()
+    off = _i32(expert_offsets).contiguous()
+    E, I2, H = w_fc.shape
+    if x.shape[1] != H or w_fc.dtype != x.dtype or I2 % 2:
+        raise ValueError("x must be (T, H), w_fc (E, 2I, H), same dtype")
+    L = ss.numel()
+    if x.shape[0] * k != L:
+        raise ValueError("x must have L / k rows")
+    if x.dtype in (torch.float16, torch.bfloat16) and L > 0:
+        lib = _lib.load()
+        act = torch.empty((L, I2 // 2), dtype=x.dtype, device=x.device)
+        h = torch.empty((L, I2), dtype=x.dtype, device=x.device)
+        with _stage("up_swiglu"):
+            rc = lib.mi_moe_up_swiglu_keep(_ptr(x), _ptr(w_fc), _ptr(act), _ptr(h), _ptr(ss), _ptr(off), L, H, I2 // 2,
+                                           E, k, _code(x.dtype), _stream())
+        if rc == 0:
+            return act, h
+        if rc not in (_lib.MI_MOE_EUNSUPPORTED, _lib.MI_MOE_EALIGN):
+            check(rc)
+    h = scattered_gemm(x, w_fc, k, ss, off, False, True)
+    return swiglu_forward(h), h
+
+
 def _fp8_unit_rows(glu: bool) -> int:
     return 16 if glu else 32
 

@@ -258,6 +258,20 @@ int mi_moe_up_swiglu_ws(const void* x, const void* w_fc, void* act_out, const in
                         void* ws, size_t ws_bytes, mi_moe_stream_t stream);
 
 /*
+ * The same up-projection for training: next to act_out it writes the (L, 2I) pre-activation h, which the backward
+ * needs (SwiGLU's derivative and the weight gradient), from the same accumulators -- one launch and one pass over h
+ * less than mi_moe_scattered_gemm followed by mi_moe_swiglu_forward.  h is rounded to `dtype` and act_out is formed
+ * from the ROUNDED halves, as mi_moe_swiglu_forward forms it from the stored h (what GLUActivation does to the
+ * output of the grouped GEMM, glu.py:42-43), with this kernel's reciprocal in place of that kernel's division.
+ * F16 / BF16 and the shapes and loads for which cfg -1 picks the persistent tile kernel (H % 32 == 0, H >= 128,
+ * I % 8 == 0, E <= 256, on average >= 192 rows per expert); MI_MOE_EUNSUPPORTED otherwise, and the caller makes
+ * the two calls.  h_out 16-byte aligned.
+ */
+int mi_moe_up_swiglu_keep(const void* x, const void* w_fc, void* act_out, void* h_out, const int32_t* sorted_scattered,
+                          const int32_t* expert_offsets, int L, int H, int I, int E, int k, int dtype,
+                          mi_moe_stream_t stream);
+
+/*
  * Gate-weighted combine:  y[t, :] = sum_j gates[t, j] * o[t*k + j, :]   (fp32 accumulation).
  * Replaces: the gates contraction inside scattered_experts(gates=...) (moe.py:282-290).
  *   o (T*k, H), gates (T, k), y (T, H) of `dtype`.

@@ -175,6 +175,46 @@ def test_grouped_wgrad(device, dtype, L, E, M, N, rows_other, gather):
         assert not got[e].any()
 
 
+KEEP_CASES = [
+    # counts per expert, H, I
+    ([5000, 5000, 5000, 5000], 1536, 512),          # interior tiles, a partly filled last round
+    ([1, 9000, 0, 300, 12000, 257], 1024, 520),     # ragged experts (row tails), ragged last column tile
+    ([700, 0, 650, 900], 256, 128),                 # few tiles, short contraction
+    ([40, 30, 20, 10], 256, 64),                    # too few rows per expert for the tile kernel: the two-call path
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("counts,H,I", KEEP_CASES)
+def test_up_swiglu_keep(device, dtype, counts, H, I):
+    """The training up-projection (activation and pre-activation from one launch) against the two calls it stands
+    for: the pre-activation bit for bit (same accumulators, same rounding), the activation formed from the rounded
+    pre-activation, equal up to the last place (a reciprocal where the element-wise kernel divides)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(sum(counts) + H)
+    E, L, k = len(counts), sum(counts), 2
+    T = L // k
+    assert T * k == L
+    off = torch.tensor(counts).cumsum(0).to(torch.int32).to(device)
+    ss = torch.randperm(L, generator=g).to(torch.int32).to(device)
+    x = torch.randn(T, H, generator=g).to(dtype).to(device)
+    w = (torch.randn(E, 2 * I, H, generator=g) * 0.05).to(dtype).to(device)
+    print(f"up_swiglu_keep {dtype} counts={counts} H={H} I={I}", flush=True)
+    act, h = ops.up_swiglu_keep(x, w, k, ss, off)
+    h_ref = ops.scattered_gemm(x, w, k, ss, off, False, True)
+    act_ref = ops.swiglu_forward(h_ref)
+    assert h.shape == (L, 2 * I) and act.shape == (L, I)
+    assert torch.equal(h, h_ref)
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    diff = (act.float() - act_ref.float()).abs()
+    assert bool((diff <= act_ref.float().abs() * 2 * eps + 1e-6).all())
+    assert (act != act_ref).float().mean().item() < 0.02
+    # and against fp32 arithmetic on the same rounded h
+    hf = h_ref.float()
+    ref = hf[:, :I] * torch.nn.functional.silu(hf[:, I:])
+    assert_close_scaled(act, ref, dtype, rtol=2e-2, atol=2e-2, what="up_swiglu_keep")
+
+
 def test_grouped_wgrad_is_deterministic(device):
     g = torch.Generator().manual_seed(5)
     L, E, M, N = 9000, 6, 256, 512
