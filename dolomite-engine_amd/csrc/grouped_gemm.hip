@@ -1087,6 +1087,11 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   T* __restrict__ out = static_cast<T*>(a.out);
   static_assert(NW * EPI_BYTES <= STAGE_BYTES, "epilogue scratch must fit the free ring stage");
   constexpr int RPP = 64 / EPI_CPR;  // rows per read-back pass
+  static_assert(RPP == 8, "read-back row order below");
+  // Row of the 32-row block that read-back instruction `it` takes for this lane: instruction 0 the even rows of
+  // the first sixteen, instruction 1 the odd ones, then the second sixteen.  All rows of an instruction have the
+  // same parity, which is what lets the epilogue's writes use both 8-byte halves of a 16-byte chunk (see there).
+  auto rb_row = [&](int it) { return 16 * (it >> 1) + 2 * (lane / EPI_CPR) + (it & 1); };
   constexpr int MP = MB / EPI_MB;    // 32-row passes over the wave's token rows
   // Destination rows of everything this lane will store in a tile's epilogue.  With scattered output they are
   // fetched one tile ahead (next to the gather indices of the tile after), so that the epilogue does not start
@@ -1097,20 +1102,20 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
   auto load_out_rows = [&](const TileCoord& tc, OutRows& o) {
     // (rows past the expert's end are never stored: with scattered output they read the index of its last row, so
     // that the loads need no predicates)
-    const int row0 = tc.row_begin + wm * WTM + lane / EPI_CPR;
+    const int row0 = tc.row_begin + wm * WTM;
     if (a.scatter) {
 #pragma unroll
       for (int mp = 0; mp < MP; ++mp)
 #pragma unroll
         for (int it = 0; it < 32 / RPP; ++it) {
-          const int row = row0 + mp * 32 + it * RPP;
+          const int row = row0 + mp * 32 + rb_row(it);
           o.r[mp][it] = a.sorted_scattered[row < tc.row_end ? row : tc.row_end - 1];
         }
     } else {
 #pragma unroll
       for (int mp = 0; mp < MP; ++mp)
 #pragma unroll
-        for (int it = 0; it < 32 / RPP; ++it) o.r[mp][it] = row0 + mp * 32 + it * RPP;
+        for (int it = 0; it < 32 / RPP; ++it) o.r[mp][it] = row0 + mp * 32 + rb_row(it);
     }
   };
   // INTERIOR: every row and column of the tile exists (all tiles but an expert's last row tile and a ragged last
@@ -1134,8 +1139,12 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
     // the ring stage consumed last is free until the next tile's first memory phase refills it (the tile loop
     // puts a barrier between this epilogue and that refill)
     unsigned char* scratch = smem_raw + ((g + NSTAGE - 1) & (NSTAGE - 1)) * STAGE_BYTES + wave * EPI_BYTES;
-    // scratch row r keeps its EPI_CPR 16-byte chunks at slots chunk ^ swz(r): the 8-byte writes of a
-    // wave and the 16-byte read-back both spread over all banks
+    // Scratch row r (128 bytes: the full width of the 32 banks) keeps its 16-byte chunks at slots chunk ^ swz(r),
+    // and odd rows keep the two 8-byte halves of every chunk swapped: the sixteen lanes that write together hold
+    // sixteen different rows and the same 8 bytes of each, and land in sixteen different bank pairs (with the chunk
+    // swizzle alone rows 2j and 2j + 1 collided on every write: 1000 conflict cycles per plain tile, now 500 --
+    // off the critical path either way, the layer's time did not move).
+    // The read-back takes rows of one parity per instruction and swaps the halves of the odd ones by naming.
     auto swz = [](int r) { return (r >> 1) & 7; };
     const auto& orow_of = orows.r;
 #pragma unroll
@@ -1173,10 +1182,10 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
             const int colp = ob * MT + fhalf * 4;  // column inside the pass
             const u32x2 p = {pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3])};
             *reinterpret_cast<u32x2*>(scratch + srow * (EPI_COLS * 2) + (((colp >> 3) ^ swz(srow)) * 16) +
-                                      ((colp >> 2) & 1) * 8) = p;
+                                      (((colp >> 2) ^ srow) & 1) * 8) = p;
           }
         }
-        // read back: lane -> row it*RPP + lane/EPI_CPR, 16-byte chunk lane%EPI_CPR
+        // read back: lane -> row rb_row(it), 16-byte chunk lane%EPI_CPR
         const int cchunk = lane % EPI_CPR;
         // column of the result (the predicate's), and of what this form writes
         const int col = tc.nt * BN + (GLU ? wn * (WTN / 2) : wn * WTN) + og * EPI_COLS + cchunk * 8;
@@ -1192,15 +1201,16 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_persistent_kernel(Ge
           u32x4 vals[RB];
 #pragma unroll
           for (int j = 0; j < RB; ++j) {
-            const int r = (it0 + j) * RPP + lane / EPI_CPR;
-            vals[j] = *reinterpret_cast<const u32x4*>(scratch + r * (EPI_COLS * 2) + ((cchunk ^ swz(r)) * 16));
+            const int r = rb_row(it0 + j);
+            const u32x4 v = *reinterpret_cast<const u32x4*>(scratch + r * (EPI_COLS * 2) + ((cchunk ^ swz(r)) * 16));
+            vals[j] = ((it0 + j) & 1) ? u32x4{v[2], v[3], v[0], v[1]} : v;
           }
 #pragma unroll
           for (int j = 0; j < RB; ++j) asm volatile("" : "+v"(vals[j]));
 #pragma unroll
           for (int j = 0; j < RB; ++j) {
             const int it = it0 + j;
-            const int r = it * RPP + lane / EPI_CPR;
+            const int r = rb_row(it);
             const int row = tc.row_begin + wm * WTM + mp * 32 + r;
             if (INTERIOR || (row < tc.row_end && col < a.N)) {
               int orow = orow_of[mp][it];
