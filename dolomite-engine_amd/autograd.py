@@ -173,6 +173,24 @@ class SwitchAuxLoss(torch.autograd.Function):
         return ops.aux_loss_backward(logits.detach(), loss_w, grad), None
 
 
+_ONE_EXPERT_ROWS: dict = {}
+_ONE_EXPERT_ROWS_MAX = 16
+
+
+def _one_expert_rows(T: int, device: torch.device):
+    """(sorted_scattered_idxs, expert_offsets) of one expert that owns rows 0..T-1 in order.  Read-only and kept per
+    (T, device) -- never released, so a captured graph may hold their addresses; beyond a few shapes they are made
+    per call."""
+    key = (T, device.index)
+    hit = _ONE_EXPERT_ROWS.get(key)
+    if hit is not None:
+        return hit
+    made = (torch.arange(T, dtype=torch.int32, device=device), torch.full((1,), T, dtype=torch.int32, device=device))
+    if len(_ONE_EXPERT_ROWS) < _ONE_EXPERT_ROWS_MAX:
+        _ONE_EXPERT_ROWS[key] = made
+    return made
+
+
 class FusedRouter(torch.autograd.Function):
     """MoE._compute_routing_weights (moe.py:246-257) as one differentiable function on this package's kernels:
 
@@ -197,8 +215,7 @@ class FusedRouter(torch.autograd.Function):
         if d_logits is None and d_gates is None:
             return None, None, None, None
         dl = ops.router_dlogits(logits, experts, d_gates, d_logits)
-        rows = torch.arange(T, dtype=torch.int32, device=x.device)
-        off = torch.full((1,), T, dtype=torch.int32, device=x.device)
+        rows, off = _one_expert_rows(T, x.device)
         dx = dw = None
         if ctx.needs_input_grad[0]:
             # (T, E) @ (E, H): the gate weight transposed to (H, E) is the "(out, in)" weight of one expert

@@ -385,26 +385,42 @@ __global__ __launch_bounds__(512) void grouped_wgrad_kernel(WgradArgs a) {
 // groups by their number of rows (longest first, ties in row order) and deal them to the XCDs back and forth.
 //   plan[0..8)   work counters
 //   plan[8..17)  first slot of XCD x in the list (slot 8 + 8 = one past the end)
+//   plan[17]     number of experts the reduction has to write (those with no group or with several)
 //   plan[32..)   group numbers (row order numbering, as the partial slabs and the reduction use) by slot
+//   plan[red_at..)  (expert, first group, groups) of each of those experts, in expert order
 // Up to WGRAD_PLAN_SORT groups are ranked; beyond that the groups are dealt in row order.
 #define WGRAD_PLAN_SORT 8192
 __global__ __launch_bounds__(1024) void wgrad_plan_kernel(const int32_t* __restrict__ offsets, int E, int chunk,
-                                                          int* __restrict__ plan) {
+                                                          int* __restrict__ plan, int red_at) {
   __shared__ int first[WGRAD_MAX_E + 1];  // groups in front of expert e
   __shared__ int ends[WGRAD_MAX_E];       // the offsets (one round trip to memory for all of them)
+  __shared__ int cnt[WGRAD_MAX_E];        // groups of expert e
   __shared__ int rows[WGRAD_PLAN_SORT];
   const int tid = threadIdx.x;
   if (tid < 8) plan[tid] = 0;
   for (int e = tid; e < E; e += blockDim.x) ends[e] = offsets[e];
   __syncthreads();
-  if (tid == 0) {
-    int g = 0;
-    for (int e = 0; e < E; ++e) {
-      first[e] = g;
-      const int n = ends[e] - (e > 0 ? ends[e - 1] : 0);
-      g += (n + chunk - 1) / chunk;
+  // groups of expert e, then every expert adds up the ones in front of it by itself (E <= 256: no scan needed)
+  for (int e = tid; e < E; e += blockDim.x) {
+    const int n = ends[e] - (e > 0 ? ends[e - 1] : 0);
+    cnt[e] = (n + chunk - 1) / chunk;
+  }
+  __syncthreads();
+  for (int e = tid; e <= E; e += blockDim.x) {
+    int g = 0, nred = 0;
+    for (int i = 0; i < e; ++i) {
+      const int c = cnt[i];
+      g += c;
+      nred += c != 1 ? 1 : 0;
     }
-    first[E] = g;
+    first[e] = g;
+    if (e == E) {
+      plan[17] = nred;
+    } else if (cnt[e] != 1) {  // not written by the main kernel
+      plan[red_at + 3 * nred] = e;
+      plan[red_at + 3 * nred + 1] = g;
+      plan[red_at + 3 * nred + 2] = cnt[e];
+    }
   }
   __syncthreads();
   const int G = first[E];
@@ -449,36 +465,51 @@ __global__ __launch_bounds__(1024) void wgrad_plan_kernel(const int32_t* __restr
 }
 
 // dW[e] = sum of expert e's partial slabs in group order, rounded once (experts with several groups); zeros for an
-// expert without rows
+// expert without rows.  blockIdx.y walks the plan's list of such experts (without a plan -- a call with no rows at
+// all -- every expert gets zeros); the blocks of an entry stride over the expert's 8-value chunks, four slabs'
+// loads in flight per chunk.
 template <typename T>
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ partial,
-                                                           const int32_t* __restrict__ offsets, T* __restrict__ dw,
-                                                           int E, long mn, int chunk) {
-  const int e = blockIdx.y;
-  int first = 0, prev = 0;
-  for (int i = 0; i < e; ++i) {
-    const int end = offsets[i];
-    first += (end - prev + chunk - 1) / chunk;
-    prev = end;
+                                                           const int* __restrict__ plan, int red_at,
+                                                           T* __restrict__ dw, long mn) {
+  int e = blockIdx.y, first = 0, count = 0;
+  if (plan != nullptr) {
+    if ((int)blockIdx.y >= plan[17]) return;
+    const int* entry = plan + red_at + 3 * blockIdx.y;
+    e = entry[0];
+    first = entry[1];
+    count = entry[2];
   }
-  const int count = (offsets[e] - prev + chunk - 1) / chunk;
-  if (count == 1) return;  // written by the main kernel
   const long n8 = mn / 8;
+  const float* base = partial + (size_t)first * mn;
+  T* out = dw + (size_t)e * mn;
   for (long id = (long)blockIdx.x * 256 + threadIdx.x; id < n8; id += (long)gridDim.x * 256) {
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-    for (int g = 0; g < count; ++g) {
-      const float* p = partial + (size_t)(first + g) * mn + id * 8;
-      const f32x4 v0 = *reinterpret_cast<const f32x4*>(p);
-      const f32x4 v1 = *reinterpret_cast<const f32x4*>(p + 4);
-      s0 += v0;
-      s1 += v1;
+    const float* p = base + id * 8;
+    int g = 0;
+    for (; g + 4 <= count; g += 4) {
+      f32x4 v[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + (size_t)(g + j) * mn));
+        v[2 * j + 1] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + (size_t)(g + j) * mn + 4));
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        s0 += v[2 * j];
+        s1 += v[2 * j + 1];
+      }
+    }
+    for (; g < count; ++g) {
+      s0 += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + (size_t)g * mn));
+      s1 += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + (size_t)g * mn + 4));
     }
     u32x4 o;
     o[0] = pack2<T>(s0[0], s0[1]);
     o[1] = pack2<T>(s0[2], s0[3]);
     o[2] = pack2<T>(s1[0], s1[1]);
     o[3] = pack2<T>(s1[2], s1[3]);
-    *reinterpret_cast<u32x4*>(dw + (size_t)e * mn + id * 8) = o;
+    *reinterpret_cast<u32x4*>(out + id * 8) = o;
   }
 }
 
@@ -498,13 +529,14 @@ static int wgrad_chunk(int L, int M, int N) {
 }
 
 static long wgrad_max_groups(int L, int E, int chunk) { return (long)L / chunk + (E < L ? E : L); }
-static size_t wgrad_plan_bytes(long groups) { return ((size_t)(32 + groups) * sizeof(int) + 255) / 256 * 256; }
+static size_t wgrad_plan_bytes(long groups, int E) { return ((size_t)(32 + groups + 3 * (long)E) * sizeof(int) + 255) / 256 * 256; }
 
 extern "C" size_t mi_moe_grouped_wgrad_workspace_bytes(int L, int E, int M, int N) {
   if (L < 1 || E < 1 || M < 1 || N < 1) return 0;
-  // [partial slabs][plan: 32 ints (work counters, first slots) + one int per group, padded to 256 bytes]
+  // [partial slabs][plan: 32 ints (work counters, first slots) + one int per group + three per expert, padded to
+  // 256 bytes]
   const long groups = wgrad_max_groups(L, E, wgrad_chunk(L, M, N));
-  return (size_t)groups * (size_t)M * (size_t)N * sizeof(float) + wgrad_plan_bytes(groups);
+  return (size_t)groups * (size_t)M * (size_t)N * sizeof(float) + wgrad_plan_bytes(groups, E);
 }
 
 extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const void* b, const int32_t* b_idx,
@@ -530,10 +562,12 @@ extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const v
   g.next_item = nullptr;
   g.L = L; g.M = M; g.N = N; g.E = E;
   g.chunk = wgrad_chunk(L, M, N);
+  const long max_groups = wgrad_max_groups(L, E, g.chunk);
+  const int red_at = (int)(32 + max_groups);
   if (L > 0) {
     g.next_item = reinterpret_cast<int*>(static_cast<unsigned char*>(workspace) +
-                                         (size_t)wgrad_max_groups(L, E, g.chunk) * (size_t)M * (size_t)N * sizeof(float));
-    hipLaunchKernelGGL(wgrad_plan_kernel, dim3(1), dim3(1024), 0, s, expert_offsets, E, g.chunk, g.next_item);
+                                         (size_t)max_groups * (size_t)M * (size_t)N * sizeof(float));
+    hipLaunchKernelGGL(wgrad_plan_kernel, dim3(1), dim3(1024), 0, s, expert_offsets, E, g.chunk, g.next_item, red_at);
   }
   g.m_tiles = mi_ceil_div(M, 256);
   g.n_tiles = mi_ceil_div(N, 256);
@@ -541,25 +575,25 @@ extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const v
   int cus = 0;
   int rc = mi_cu_count(&cus);
   if (rc != MI_MOE_OK) return rc;
-  const long max_items = wgrad_max_groups(L, E, g.chunk) * g.m_tiles * g.n_tiles;
+  const long max_items = max_groups * g.m_tiles * g.n_tiles;
   long grid = cus < max_items ? cus : max_items;
   grid = (grid + 7) / 8 * 8;
   long rblocks = (mn / 8 + 255) / 256;
-  if (rblocks > 4096) rblocks = 4096;
+  if (rblocks > 256) rblocks = 256;
   if (dtype == MI_MOE_BF16) {
     auto kern = grouped_wgrad_kernel<bf16_t>;
     static std::atomic<uint64_t> lds_ok{0};
     if ((rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok)) != MI_MOE_OK) return rc;
     if (L > 0) hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, s, g);
     hipLaunchKernelGGL((wgrad_reduce_kernel<bf16_t>), dim3((unsigned)rblocks, (unsigned)E), dim3(256), 0, s, g.partial,
-                       expert_offsets, static_cast<bf16_t*>(dw), E, mn, g.chunk);
+                       g.next_item, red_at, static_cast<bf16_t*>(dw), mn);
   } else {
     auto kern = grouped_wgrad_kernel<f16_t>;
     static std::atomic<uint64_t> lds_ok{0};
     if ((rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok)) != MI_MOE_OK) return rc;
     if (L > 0) hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, s, g);
     hipLaunchKernelGGL((wgrad_reduce_kernel<f16_t>), dim3((unsigned)rblocks, (unsigned)E), dim3(256), 0, s, g.partial,
-                       expert_offsets, static_cast<f16_t*>(dw), E, mn, g.chunk);
+                       g.next_item, red_at, static_cast<f16_t*>(dw), mn);
   }
   return mi_launch_status();
 }
