@@ -210,8 +210,9 @@ __global__ __launch_bounds__(256) void router_fused_kernel(const T* __restrict__
 // 16-byte bank groups) and then walks 16-token groups, one per wave and turn; x streams through a register ring
 // DEPTH K steps deep (3 with eight waves: about 48 KB in flight per CU), and only the ceil(E / 16) expert blocks that exist are
 // multiplied.
-// With fewer than eight groups per CU the launch uses fewer waves per workgroup (so that every CU takes part)
-// and a deeper ring per wave (DEPTH 6) to keep as many bytes in flight.
+// With fewer than eight groups per CU fewer waves per workgroup walk groups (so that every CU takes part), with a
+// deeper ring per wave (DEPTH 6) to keep as many bytes in flight; the workgroup still has eight waves for the copy
+// of the weights (one wave alone took 20 us over it: 29 us for this kernel at 1024 - 4096 tokens).
 #define ROUTER_LDS_WAVES 8
 // NORM folds the RMSNorm in front of the layer (ln_2 of the transformer block, mixins/dense/layer.py:58-59;
 // normalization.py:19-34 = torch.nn.RMSNorm) into the same kernel: a group's rows are streamed twice, first for
@@ -225,25 +226,24 @@ struct RouterNorm {
 };
 
 // `chunk_hist` (or null): the first pass of the expert sort (routing.hip) done here.  The groups a workgroup takes
-// in one turn are consecutive -- a chunk of blockDim / 64 * 16 tokens -- so the workgroup counts the experts its
+// in one turn are consecutive -- a chunk of nwaves * 16 tokens -- so the workgroup counts the experts its
 // waves select in LDS and writes chunk_hist[e * nchunks + chunk], the layout the sort's scan pass reads; the sort
 // then needs neither its histogram launch nor that launch's read of the expert ids.
 template <typename T, int DEPTH, bool NORM>
 __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ gw, const float* __restrict__ bias, int Trows, int H, int E, int k,
     T* __restrict__ logits_out, T* __restrict__ gates, int32_t* __restrict__ idx, RouterNorm norm,
-    int32_t* __restrict__ chunk_hist, int nchunks) {
+    int32_t* __restrict__ chunk_hist, int nchunks, int nwaves) {
   typedef typename RMfma<T>::vec frag_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char wlds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, q = lane >> 4;
   const int pitch = H * (int)sizeof(T) + 16;
-  // ---- gate weights -> LDS (16-byte pieces; H % 16 == 0 is checked on the host) ----
-  const int nwaves = blockDim.x >> 6;
+  // the first `nwaves` waves walk token groups; the others only help to copy the weights (and keep the barriers)
   const int nsteps = (H + 63) >> 6;
   const int ngroups = (Trows + 15) >> 4;
   const int stride = gridDim.x * nwaves;
-  int grp = blockIdx.x * nwaves + wave;
+  int grp = wave < nwaves ? blockIdx.x * nwaves + wave : ngroups;
 
   // x ring of the wave's current group; the first DEPTH steps of a group are requested before the previous
   // group's epilogue (for the first group: before the weights are copied), so their latency is hidden
@@ -632,8 +632,19 @@ static int router_splits(int T_, int H) {
   return splits;
 }
 
-static size_t router_ws_bytes(int T_, int H) {
-  if (T_ <= 0 || T_ > 1024) return 0;
+// gate weights (16 bits an element) fit in LDS next to the per-expert words of the LDS-resident kernel
+static bool router_lds_fits(int H, int E) { return (size_t)E * ((size_t)H * 2 + 16) <= 156u * 1024u; }
+
+// The few-token forms (K split across waves or workgroups) are used up to ROUTER_FEW_TOKENS tokens, and up to 1024
+// where the LDS-resident kernel does not take the gate weights.  Every entry point applies the same rule, so that
+// the router gives the same bits whichever of them a caller uses.  Measured, router + sort as the layer calls them,
+// hidden size 1536, 40 experts, top-8: few-token form 22.5 / 26 / 35 / 43 us at 384 / 512 / 768 / 1024 tokens (its
+// one-block sort is what grows), LDS-resident kernel + scan + scatter 24.6 us from 192 to 2048 tokens.
+#define ROUTER_FEW_TOKENS 384
+static bool router_few_tokens(int T_, int H, int E) { return T_ <= (router_lds_fits(H, E) ? ROUTER_FEW_TOKENS : 1024); }
+
+static size_t router_ws_bytes(int T_, int H, int E) {
+  if (T_ <= 0 || !router_few_tokens(T_, H, E)) return 0;
   return (size_t)router_splits(T_, H) * mi_ceil_div(T_, 16) * 4 * 64 * sizeof(f32x4);
 }
 
@@ -677,16 +688,16 @@ static int launch_router_lds(const void* x, const void* gw, const float* bias, i
   static std::atomic<uint64_t> lds_ok[2];  // the LDS size varies with E and H: opt in to the most it can be
   rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok[waves > 4 ? 1 : 0]);
   if (rc != MI_MOE_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(waves * 64), lds + (size_t)E * sizeof(int), s, static_cast<const T*>(x),
-                     static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out),
-                     static_cast<T*>(gates), idx, norm, chunk_hist, nchunks);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(ROUTER_LDS_WAVES * 64), lds + (size_t)E * sizeof(int), s,
+                     static_cast<const T*>(x), static_cast<const T*>(gw), bias, T_, H, E, k,
+                     static_cast<T*>(logits_out), static_cast<T*>(gates), idx, norm, chunk_hist, nchunks, waves);
   return mi_launch_status();
 }
 
 template <typename T>
 static int launch_router(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
                          void* logits_out, void* gates, int32_t* idx, hipStream_t s) {
-  if (T_ <= 1024) {  // fewer than 4 workgroups' worth of tokens for the streaming kernel: split K instead
+  if (router_few_tokens(T_, H, E)) {  // split K across the waves of a workgroup instead
     hipLaunchKernelGGL((router_fused_small_kernel<T>), dim3(mi_ceil_div(T_, 16)), dim3(1024), 0, s,
                        static_cast<const T*>(x), static_cast<const T*>(gw), bias, T_, H, E, k,
                        static_cast<T*>(logits_out), static_cast<T*>(gates), idx);
@@ -706,9 +717,10 @@ static int launch_router(const void* x, const void* gw, const float* bias, int T
   return mi_launch_status();
 }
 
+// Router + sort in two launches (split K, the finishing launch sorts in its last workgroup).
 // [partial logits][ticket, padded to 256 bytes]
-static size_t router_sort_ws_bytes(int T_, int H, int k) {
-  const size_t base = router_ws_bytes(T_, H);
+static size_t router_sort_ws_bytes(int T_, int H, int E, int k) {
+  const size_t base = router_ws_bytes(T_, H, E);
   if (base == 0 || (long)T_ * k > SORT_SINGLE_BLOCK_MAX) return 0;
   return base + 256;
 }
@@ -720,7 +732,7 @@ static int launch_router_splitk_sort(const void* x, const void* gw, const float*
   const int splits = router_splits(T_, H);
   const int steps_per_split = mi_ceil_div(mi_ceil_div(H, 64), splits);
   const int groups = mi_ceil_div(T_, 16);
-  unsigned* ticket = reinterpret_cast<unsigned*>(static_cast<unsigned char*>(ws) + router_ws_bytes(T_, H));
+  unsigned* ticket = reinterpret_cast<unsigned*>(static_cast<unsigned char*>(ws) + router_ws_bytes(T_, H, E));
   hipLaunchKernelGGL((router_splitk_partial_kernel<T>), dim3(groups, splits), dim3(ROUTER_SPLIT_WAVES * 64), 0, s,
                      static_cast<const T*>(x), static_cast<const T*>(gw), T_, H, E, steps_per_split,
                      static_cast<f32x4*>(ws), ticket);
@@ -740,8 +752,8 @@ int mi_sort_after_hist(const int32_t* topk_idx, int L, int E, int chunk, int32_t
                        int32_t* sorted_scattered, int32_t* expert_offsets, int32_t* ws, hipStream_t s);
 
 static bool router_hist_shape(int T_, int H, int E, int k, int* chunk_tokens, int* nchunks) {
-  if (T_ <= 1024 || (long)T_ * k > 0x7fffffffL - 8192) return false;
-  if ((size_t)E * ((size_t)H * 2 + 16) > 156u * 1024u) return false;  // gate weights must fit in LDS
+  if (router_few_tokens(T_, H, E) || (long)T_ * k > 0x7fffffffL - 8192) return false;
+  if (!router_lds_fits(H, E)) return false;
   int blocks = 0, waves = 0;
   if (router_lds_shape(T_, &blocks, &waves) != MI_MOE_OK) return false;
   *chunk_tokens = waves * 16;
@@ -751,7 +763,7 @@ static bool router_hist_shape(int T_, int H, int E, int k, int* chunk_tokens, in
 
 extern "C" size_t mi_moe_router_fused_sort_workspace_bytes(int T, int H, int E, int k) {
   if (T < 1 || H < 1 || k < 1 || E < 1) return 0;
-  const size_t small = router_sort_ws_bytes(T, H, k);
+  const size_t small = router_sort_ws_bytes(T, H, E, k);
   if (small) return small;
   int chunk_tokens = 0, nchunks = 0;
   if (E > 64 || k > ROUTER_KMAX || H % 16 != 0 || !router_hist_shape(T, H, E, k, &chunk_tokens, &nchunks)) return 0;
@@ -771,7 +783,7 @@ extern "C" int mi_moe_router_fused_sort(const void* x, const void* gate_w, const
   if (!ws || ws_bytes < need) return MI_MOE_EWORKSPACE;
   if (!mi_aligned(x, 16) || !mi_aligned(gate_w, 16) || !mi_aligned(ws, 16)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (router_sort_ws_bytes(T, H, k) != 0) {
+  if (router_sort_ws_bytes(T, H, E, k) != 0) {
     if (dtype == MI_MOE_BF16)
       return launch_router_splitk_sort<bf16_t>(x, gate_w, bias, T, H, E, k, logits_out, gates_out, idx_out,
                                                sorted_expert, sorted_scattered, expert_offsets, ws, s);
@@ -793,8 +805,7 @@ extern "C" int mi_moe_router_fused_sort(const void* x, const void* gate_w, const
 }
 
 extern "C" size_t mi_moe_router_fused_workspace_bytes(int T, int H, int E) {
-  (void)E;
-  return (T < 0 || H < 1) ? 0 : router_ws_bytes(T, H);
+  return (T < 0 || H < 1 || E < 1) ? 0 : router_ws_bytes(T, H, E);
 }
 
 // router_general.hip: fp32, 65 .. 256 experts, k up to 64
@@ -814,7 +825,7 @@ extern "C" int mi_moe_router_fused(const void* x, const void* gate_w, const floa
   if (!mi_aligned(x, 16) || !mi_aligned(gate_w, 16)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (!streaming) return mi_router_general(x, gate_w, bias, T, H, E, k, dtype, logits_out, gates_out, idx_out, s);
-  const size_t need = router_ws_bytes(T, H);
+  const size_t need = router_ws_bytes(T, H, E);
   if (ws != nullptr && need > 0) {  // few tokens and a workspace: K split across workgroups
     if (ws_bytes < need) return MI_MOE_EWORKSPACE;
     if (!mi_aligned(ws, 16)) return MI_MOE_EALIGN;

@@ -276,7 +276,9 @@ def test_rmsnorm_router_fused_unsupported_shapes(device):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,H,E,k,bias", [(1, 64, 8, 2, False), (15, 32, 8, 8, False), (64, 4096, 64, 6, False),
                                           (200, 256, 40, 8, True), (1000, 1024, 32, 8, False), (1024, 512, 64, 8, True),
-                                          (130, 48, 5, 1, False),
+                                          (130, 48, 5, 1, False), (384, 1536, 40, 8, True), (1024, 4096, 64, 6, False),
+                                          # just past the few-token form where the gate weights fit in LDS
+                                          (385, 1536, 40, 8, True), (768, 1024, 32, 8, False),
                                           # many tokens: the router counts the experts per chunk for the sort
                                           (1025, 64, 8, 2, False), (2500, 256, 40, 8, True), (4099, 512, 64, 6, False),
                                           (16384, 1024, 32, 8, False), (32768, 1536, 40, 8, True),
@@ -311,6 +313,9 @@ def test_router_fused_sort_limits(device):
     assert not ops.router_fused_sort_supported(torch.zeros(2048, 4096, dtype=torch.bfloat16, device=device), 64, 2)  # gate weights beyond LDS
     assert not ops.router_fused_sort_supported(x[:1024], 64, 9)  # k beyond the fused router
     assert ops.router_fused_sort_supported(x[:1024], 64, 8)      # 8192 slots: the one-block sort's limit
+    big = torch.zeros(1025, 4096, dtype=torch.bfloat16, device=device)
+    assert ops.router_fused_sort_supported(big[:1024], 64, 6)    # gate weights beyond LDS: the few-token form up to 1024
+    assert not ops.router_fused_sort_supported(big, 64, 6)
 
 
 @pytest.mark.parametrize("seed", [1, 2, 3])
