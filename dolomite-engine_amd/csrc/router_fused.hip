@@ -3,7 +3,7 @@
 // results (and optionally the logits) written.
 // Stands in for MoE._compute_routing_weights, lm_engine/hf_models/modeling_utils/mlp_blocks/moe.py:246-257.
 //
-// HBM-bound on reading x.  A wavefront owns TG groups of 16 tokens and all (<= 64) experts:
+// HBM-bound on reading x.  A wavefront works on groups of 16 tokens and all (<= 64) experts:
 //   * v_mfma_f32_16x16x32 with the gate weights as operand A (16 experts x 32 k) and the tokens as
 //     operand B, so lane (r = l%16, q = l/16) ends with logits of token r for experts 16*eb + 4q + i;
 //   * lane (r, q) streams 16 consecutive k of its token row per 64-wide K step (two dwordx4), so the four
@@ -130,82 +130,8 @@ __device__ __forceinline__ void router_epilogue(const f32x4 (&acc)[4], int t, bo
   }
 }
 
-template <typename T, int TG>
-__global__ __launch_bounds__(256) void router_fused_kernel(const T* __restrict__ x, const T* __restrict__ gw,
-                                                           const float* __restrict__ bias, int Trows, int H, int E,
-                                                           int k, T* __restrict__ logits_out, T* __restrict__ gates,
-                                                           int32_t* __restrict__ idx) {
-  typedef typename RMfma<T>::vec frag_t;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r = lane & 15, q = lane >> 4;
-  const int tok0 = (blockIdx.x * 4 + wave) * (16 * TG);
-  if (tok0 >= Trows) return;
-
-  const T* xrow[TG];
-#pragma unroll
-  for (int g = 0; g < TG; ++g) {
-    int t = tok0 + g * 16 + r;
-    if (t > Trows - 1) t = Trows - 1;
-    xrow[g] = x + (size_t)t * H;
-  }
-  const T* wrow[4];
-#pragma unroll
-  for (int eb = 0; eb < 4; ++eb) {
-    int e = eb * 16 + r;
-    if (e > E - 1) e = E - 1;
-    wrow[eb] = gw + (size_t)e * H;
-  }
-
-  f32x4 acc[4][TG];
-#pragma unroll
-  for (int eb = 0; eb < 4; ++eb)
-#pragma unroll
-    for (int g = 0; g < TG; ++g) acc[eb][g] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-#pragma unroll 2
-  for (int k0 = 0; k0 < H; k0 += 64) {
-    const int kpos = k0 + q * 16;
-    const bool valid = kpos < H;
-    u32x4 xa[TG][2], wa[4][2];
-#pragma unroll
-    for (int g = 0; g < TG; ++g) {
-      xa[g][0] = xa[g][1] = (u32x4){0u, 0u, 0u, 0u};
-      if (valid) {
-        xa[g][0] = *reinterpret_cast<const u32x4*>(xrow[g] + kpos);
-        xa[g][1] = *reinterpret_cast<const u32x4*>(xrow[g] + kpos + 8);
-      }
-    }
-#pragma unroll
-    for (int eb = 0; eb < 4; ++eb) {
-      wa[eb][0] = wa[eb][1] = (u32x4){0u, 0u, 0u, 0u};
-      if (valid) {
-        wa[eb][0] = *reinterpret_cast<const u32x4*>(wrow[eb] + kpos);
-        wa[eb][1] = *reinterpret_cast<const u32x4*>(wrow[eb] + kpos + 8);
-      }
-    }
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int eb = 0; eb < 4; ++eb)
-#pragma unroll
-        for (int g = 0; g < TG; ++g)
-          acc[eb][g] = RMfma<T>::run(__builtin_bit_cast(frag_t, wa[eb][h]), __builtin_bit_cast(frag_t, xa[g][h]),
-                                     acc[eb][g]);
-  }
-
-  // ---- epilogue: round, bias, optional logits store, top-k, softmax ---------------------------
-#pragma unroll
-  for (int g = 0; g < TG; ++g) {
-    const int t = tok0 + g * 16 + r;
-    f32x4 a4[4];
-#pragma unroll
-    for (int eb = 0; eb < 4; ++eb) a4[eb] = acc[eb][g];
-    router_epilogue<T>(a4, t, t < Trows, q, bias, E, k, logits_out, gates, idx);
-  }
-}
-
-// Many tokens, gate weights held in LDS.  The kernel above re-reads the gate weights (E x H) from L2 for every
-// 32 tokens -- more bytes than x itself -- and runs four waves per CU.  Here a workgroup of eight waves copies the
+// Many tokens, gate weights held in LDS (reading the gate weights (E x H) from L2 for every few groups would move
+// more bytes than x itself).  A workgroup of eight waves copies the
 // weights into LDS once (row pitch 2H + 16 bytes: the 16 rows of a fragment read then start in 16 different
 // 16-byte bank groups) and then walks 16-token groups, one per wave and turn; x streams through a register ring
 // DEPTH K steps deep (3 with eight waves: about 48 KB in flight per CU), and only the ceil(E / 16) expert blocks that exist are
@@ -411,6 +337,107 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
     }
+  }
+}
+
+// Many tokens, gate weights too large for LDS.  A workgroup of eight waves owns ROUTER_KS_TG groups of 16 tokens;
+// wave w takes the 64-wide K steps w, w + 8, ... of all of them (two steps' loads in flight at a time), so a wave
+// walks an eighth of the row, and a step's gate-weight fragments serve every group.  The partial logits meet in
+// LDS, two groups at a time, and are added in wave order (the logits do not depend on scheduling); waves
+// 0 .. ROUTER_KS_TG - 1 then run one group's epilogue each.
+#define ROUTER_KS_WAVES 8
+#define ROUTER_KS_TG 4
+template <typename T>
+__global__ __launch_bounds__(ROUTER_KS_WAVES * 64) void router_fused_ksplit_kernel(
+    const T* __restrict__ x, const T* __restrict__ gw, const float* __restrict__ bias, int Trows, int H, int E, int k,
+    T* __restrict__ logits_out, T* __restrict__ gates, int32_t* __restrict__ idx) {
+  typedef typename RMfma<T>::vec frag_t;
+  constexpr int TG = ROUTER_KS_TG, NW = ROUTER_KS_WAVES;
+  static_assert(TG % 2 == 0 && TG <= NW, "groups are reduced in pairs, one finishing wave per group");
+  __shared__ f32x4 red[NW][2][4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int tok0 = blockIdx.x * (16 * TG);
+  const T* xrow[TG];
+#pragma unroll
+  for (int g = 0; g < TG; ++g) {
+    int t = tok0 + g * 16 + r;
+    if (t > Trows - 1) t = Trows - 1;
+    xrow[g] = x + (size_t)t * H;
+  }
+  const T* wrow[4];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb) {
+    int e = eb * 16 + r;
+    if (e > E - 1) e = E - 1;
+    wrow[eb] = gw + (size_t)e * H;
+  }
+  const int neb = (E + 15) >> 4;
+  f32x4 acc[4][TG];
+#pragma unroll
+  for (int eb = 0; eb < 4; ++eb)
+#pragma unroll
+    for (int g = 0; g < TG; ++g) acc[eb][g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  for (int k0 = wave * 64; k0 < H; k0 += 2 * NW * 64) {
+    u32x4 xa[2][TG][2], wa[2][4][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int kpos = k0 + s * NW * 64 + q * 16;
+      const bool valid = kpos < H;  // the MFMA runs on all lanes: out-of-range k contributes zeros
+#pragma unroll
+      for (int g = 0; g < TG; ++g) {
+        xa[s][g][0] = xa[s][g][1] = (u32x4){0u, 0u, 0u, 0u};
+        if (valid) {
+          xa[s][g][0] = *reinterpret_cast<const u32x4*>(xrow[g] + kpos);
+          xa[s][g][1] = *reinterpret_cast<const u32x4*>(xrow[g] + kpos + 8);
+        }
+      }
+#pragma unroll
+      for (int eb = 0; eb < 4; ++eb) {
+        wa[s][eb][0] = wa[s][eb][1] = (u32x4){0u, 0u, 0u, 0u};
+        if (valid && eb < neb) {
+          wa[s][eb][0] = *reinterpret_cast<const u32x4*>(wrow[eb] + kpos);
+          wa[s][eb][1] = *reinterpret_cast<const u32x4*>(wrow[eb] + kpos + 8);
+        }
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int eb = 0; eb < 4; ++eb)
+          if (eb < neb) {
+#pragma unroll
+            for (int g = 0; g < TG; ++g)
+              acc[eb][g] = RMfma<T>::run(__builtin_bit_cast(frag_t, wa[s][eb][h]),
+                                         __builtin_bit_cast(frag_t, xa[s][g][h]), acc[eb][g]);
+          }
+  }
+
+  f32x4 fin[4];
+#pragma unroll
+  for (int gp = 0; gp < TG / 2; ++gp) {
+    if (gp > 0) __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int eb = 0; eb < 4; ++eb) red[wave][j][eb][lane] = acc[eb][2 * gp + j];
+    __syncthreads();
+    if ((wave >> 1) == gp) {
+#pragma unroll
+      for (int eb = 0; eb < 4; ++eb) {
+        f32x4 sum = red[0][wave & 1][eb][lane];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) sum += red[w][wave & 1][eb][lane];
+        fin[eb] = sum;
+      }
+    }
+  }
+  if (wave < TG) {
+    const int t = tok0 + wave * 16 + r;
+    router_epilogue<T>(fin, t, t < Trows, q, bias, E, k, logits_out, gates, idx);
   }
 }
 
@@ -709,11 +736,9 @@ static int launch_router(const void* x, const void* gw, const float* bias, int T
     const RouterNorm none = {nullptr, nullptr, 0.f};
     return launch_router_lds<T, false>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, none, wbytes, s);
   }
-  constexpr int TG = 2;
-  dim3 grid(mi_ceil_div(T_, 4 * 16 * TG)), block(256);
-  hipLaunchKernelGGL((router_fused_kernel<T, TG>), grid, block, 0, s, static_cast<const T*>(x),
-                     static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out),
-                     static_cast<T*>(gates), idx);
+  hipLaunchKernelGGL((router_fused_ksplit_kernel<T>), dim3(mi_ceil_div(T_, 16 * ROUTER_KS_TG)),
+                     dim3(ROUTER_KS_WAVES * 64), 0, s, static_cast<const T*>(x), static_cast<const T*>(gw), bias, T_, H,
+                     E, k, static_cast<T*>(logits_out), static_cast<T*>(gates), idx);
   return mi_launch_status();
 }
 
