@@ -498,3 +498,76 @@ extern "C" int mi_moe_down_fp8(const void* act, const void* w_proj_q, const floa
   a.tiled = w_tiled != 0;
   return run_decode(a, dtype, false, static_cast<hipStream_t>(stream));
 }
+
+// ---- fp8 weights -> 16-bit weights with the channel scale folded in ----------------------------------------------
+// The kernels above stream an expert's weights once per 16 of its rows: right for decode, linear in the batch
+// beyond that.  For batches with many rows per expert the caller widens the weights once per call (w * scale in
+// fp32, one rounding) into a scratch tensor of the activation dtype and runs the tiled 16-bit grouped GEMM on it.
+// One thread per 16-byte piece of a weight row; reads either layout, writes (E, rows, K) row-major.
+template <typename T>
+__global__ __launch_bounds__(256) void fp8_dequant_kernel(const uint8_t* __restrict__ wq, const float* __restrict__ scale,
+                                                          T* __restrict__ out, long pieces, int N, int K, int glu,
+                                                          int tiled) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  const long id = (long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= pieces) return;
+  const int ppr = K >> 4;                // pieces per row
+  const long grow = id / ppr;            // row over all experts
+  const int c16 = (int)(id - grow * ppr);
+  size_t src = (size_t)id * 16;
+  if (tiled) {
+    const int R = glu ? 2 * N : N;
+    const long e = grow / R;
+    const int row = (int)(grow - e * R);
+    const int half = (glu && row >= N) ? 1 : 0;
+    const int n = row - half * N;
+    const int chw = glu ? 16 : 32;
+    const int U = (N + chw - 1) / chw;
+    const int u = n / chw;
+    const int t = n - u * chw + 16 * half;  // row inside the 32-row stage image
+    const int stage = c16 >> 3, c = c16 & 7;
+    const int slot = c ^ (((t >> 1) & 1) | (((t >> 2) & 1) << 2));
+    src = (((((size_t)e * U + u) * (size_t)(K >> 7) + stage) * 32 + t) * 8 + slot) * 16;
+  }
+  const u32x4 v = *reinterpret_cast<const u32x4*>(wq + src);
+  const float sc = scale[grow];
+  u32x4 o[2];
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(v[d], false);
+    const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(v[d], true);
+    // the product is rounded to fp32 and then to T, as `(w.float() * scale).to(T)` does: left alone, the compiler
+    // fuses product and conversion to fp16 into one fma with a zero addend (one rounding, and -0 becomes +0)
+    float p[4] = {lo[0] * sc, lo[1] * sc, hi[0] * sc, hi[1] * sc};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(p[i]));
+    o[d >> 1][(d & 1) * 2] = pack2<T>(p[0], p[1]);
+    o[d >> 1][(d & 1) * 2 + 1] = pack2<T>(p[2], p[3]);
+  }
+  u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)id * 16);
+  dst[0] = o[0];
+  dst[1] = o[1];
+}
+
+extern "C" int mi_moe_fp8_dequant(const void* w_q, const float* w_scale, void* w_out, int E, int out, int in, int glu,
+                                  int w_tiled, int dtype, mi_moe_stream_t stream) {
+  if (E < 1 || out < 1 || in < 1) return MI_MOE_ESHAPE;
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (in % 16 != 0 || (w_tiled && in % 128 != 0)) return MI_MOE_EUNSUPPORTED;
+  if (!w_q || !w_scale || !w_out) return MI_MOE_ENULL;
+  if (!mi_aligned(w_q, 16) || !mi_aligned(w_out, 16)) return MI_MOE_EALIGN;
+  const long rows = (long)E * (glu ? 2 : 1) * out;
+  const long pieces = rows * (in / 16);
+  const long blocks = (pieces + 255) / 256;
+  if (blocks > 0x7fffffffL) return MI_MOE_ESHAPE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MI_MOE_BF16)
+    hipLaunchKernelGGL((fp8_dequant_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s,
+                       static_cast<const uint8_t*>(w_q), w_scale, static_cast<bf16_t*>(w_out), pieces, out, in, glu,
+                       w_tiled);
+  else
+    hipLaunchKernelGGL((fp8_dequant_kernel<f16_t>), dim3((unsigned)blocks), dim3(256), 0, s,
+                       static_cast<const uint8_t*>(w_q), w_scale, static_cast<f16_t*>(w_out), pieces, out, in, glu,
+                       w_tiled);
+  return mi_launch_status();
+}

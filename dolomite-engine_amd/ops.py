@@ -780,10 +780,46 @@ def fp8_untile(tiled: torch.Tensor, E: int, out_rows: int, K: int, glu: bool) ->
     return w.contiguous().view(torch.float8_e4m3fn)
 
 
+# Average rows per expert from which the fp8 calls widen the weights for the call and run the tiled 16-bit kernels
+# instead: the fp8 kernels stream an expert's weights once per 16 of its rows (right for decode, linear in the
+# batch beyond), the widening is one pass over the weights whatever the batch.
+FP8_DENSE_ROWS_PER_EXPERT = 80
+
+
+def fp8_dequant(w_q: torch.Tensor, scale: torch.Tensor, in_features: int, glu: bool, dtype: torch.dtype) -> torch.Tensor:
+    """e4m3fn expert weights, row-major (E, rows, in) or tiled (:func:`fp8_tile`), with (E, rows) fp32 scales ->
+    (E, rows, in) weights of ``dtype`` (bf16 / fp16) = round(w * scale[:, :, None])."""
+    _dev(w_q, scale)
+    if w_q.dtype != torch.float8_e4m3fn or dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError("expected torch.float8_e4m3fn weights and a 16-bit result type")
+    w_q = w_q.contiguous()
+    scale = scale.to(torch.float32).contiguous()
+    E, R = scale.shape
+    K = int(in_features)
+    tiled = w_q.dim() == 1
+    lib = _lib.load()
+    if (glu and R % 2) or K % 16:
+        raise ValueError("shape mismatch")
+    out_ch = R // 2 if glu else R
+    if tiled:
+        if w_q.numel() != lib.mi_moe_fp8_tiled_bytes(E, out_ch, K, int(glu)) or w_q.numel() == 0:
+            raise ValueError("tiled weights do not match the scales and in_features")
+    elif tuple(w_q.shape) != (E, R, K):
+        raise ValueError("shape mismatch")
+    w = torch.empty((E, R, K), dtype=dtype, device=w_q.device)
+    with _stage("fp8_dequant"):
+        check(lib.mi_moe_fp8_dequant(_ptr(w_q), _ptr(scale), _ptr(w), E, out_ch, K, int(glu), int(tiled), _code(dtype),
+                                     _stream()))
+    return w
+
+
 def up_swiglu_fp8(x: torch.Tensor, w_fc_q: torch.Tensor, w_fc_scale: torch.Tensor, k: int,
-                  sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor) -> torch.Tensor:
+                  sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor,
+                  widen: bool | None = None) -> torch.Tensor:
     """As up_swiglu with e4m3fn weights and fp32 per-output-channel scales (E, 2I).  The weights are either
-    row-major (E, 2I, H) or, as a flat tensor, in the layout of :func:`fp8_tile` (``glu=True``)."""
+    row-major (E, 2I, H) or, as a flat tensor, in the layout of :func:`fp8_tile` (``glu=True``).  From
+    FP8_DENSE_ROWS_PER_EXPERT rows per expert on average the weights are widened for the call and
+    :func:`up_swiglu` runs on the copy (``widen``: True / False force either way)."""
     _dev(x, w_fc_q, w_fc_scale, sorted_scattered_idxs, expert_offsets)
     _no_grad(x)
     if w_fc_q.dtype != torch.float8_e4m3fn:
@@ -805,6 +841,8 @@ def up_swiglu_fp8(x: torch.Tensor, w_fc_q: torch.Tensor, w_fc_scale: torch.Tenso
         raise ValueError("shape mismatch")
     if x.shape[0] * k != L:
         raise ValueError("shape mismatch")
+    if (L >= FP8_DENSE_ROWS_PER_EXPERT * E if widen is None else widen) and H % 16 == 0 and L > 0:
+        return up_swiglu(x, fp8_dequant(w_fc_q, scale, H, True, x.dtype), k, ss, off)
     act = torch.empty((L, I2 // 2), dtype=x.dtype, device=x.device)
     with _stage("up_swiglu_fp8"):
         check(lib.mi_moe_up_swiglu_fp8(_ptr(x), _ptr(w_fc_q), _ptr(scale), _ptr(act), _ptr(ss), _ptr(off), L, H,
@@ -813,9 +851,11 @@ def up_swiglu_fp8(x: torch.Tensor, w_fc_q: torch.Tensor, w_fc_scale: torch.Tenso
 
 
 def down_fp8(act: torch.Tensor, w_proj_q: torch.Tensor, w_proj_scale: torch.Tensor,
-             sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor) -> torch.Tensor:
+             sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor,
+             widen: bool | None = None) -> torch.Tensor:
     """Down-projection with e4m3fn weights, row-major (E, H, I) or tiled (:func:`fp8_tile`, ``glu=False``):
-    act (L, I) grouped -> (L, H) in flat-slot order."""
+    act (L, I) grouped -> (L, H) in flat-slot order (widened weights from FP8_DENSE_ROWS_PER_EXPERT rows per expert
+    on, as in :func:`up_swiglu_fp8`)."""
     _dev(act, w_proj_q, w_proj_scale, sorted_scattered_idxs, expert_offsets)
     _no_grad(act)
     if w_proj_q.dtype != torch.float8_e4m3fn:
@@ -836,6 +876,8 @@ def down_fp8(act: torch.Tensor, w_proj_q: torch.Tensor, w_proj_scale: torch.Tens
         raise ValueError("shape mismatch")
     if ss.numel() != L:
         raise ValueError("shape mismatch")
+    if (L >= FP8_DENSE_ROWS_PER_EXPERT * E if widen is None else widen) and I % 16 == 0 and L > 0:
+        return scattered_gemm(act, fp8_dequant(w_proj_q, scale, I, False, act.dtype), 1, ss, off, True, False)
     o = torch.empty((L, H), dtype=act.dtype, device=act.device)
     with _stage("down_fp8"):
         check(lib.mi_moe_down_fp8(_ptr(act), _ptr(w_proj_q), _ptr(scale), _ptr(o), _ptr(ss), _ptr(off), L, I, H,

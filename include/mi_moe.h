@@ -380,6 +380,12 @@ int mi_moe_up_swiglu_fp8(const void* x, const void* w_fc_q, const float* w_fc_sc
 int mi_moe_down_fp8(const void* act, const void* w_proj_q, const float* w_proj_scale, void* o_out,
                     const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
                     int E, int dtype, int w_tiled, mi_moe_stream_t stream);
+/* The same weights widened to `dtype` with the channel scale folded in: w_out (E, out, in) -- (E, 2 * out, in), up
+ * rows first, with glu -- = round(w * scale[:, None]), from either layout.  For batches with many rows per expert,
+ * where the two calls above (which stream an expert's weights once per 16 of its rows) lose to the tiled 16-bit
+ * kernels on a widened copy (mi_moe_up_swiglu / mi_moe_scattered_gemm); the caller owns the copy.  in % 16 == 0. */
+int mi_moe_fp8_dequant(const void* w_q, const float* w_scale, void* w_out, int E, int out, int in, int glu,
+                       int w_tiled, int dtype, mi_moe_stream_t stream);
 
 /*
  * Diagnostics (no counterpart in the reference; nothing in the layer calls them): the pieces of the persistent

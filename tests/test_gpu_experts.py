@@ -408,11 +408,11 @@ def test_fp8_up_down(device, dtype, T, E, k, H, I):
     w_fc_q, fc_scale = oracle.quantize_fp8_per_channel(torch.randn(E, 2 * I, H, generator=g) * 0.02)
     w_pj_q, pj_scale = oracle.quantize_fp8_per_channel(torch.randn(E, H, I, generator=g) * 0.02)
     print(f"fp8 T={T} E={E} k={k} H={H} I={I} {dtype}", flush=True)
-    act = ops.up_swiglu_fp8(x.to(device), w_fc_q.to(device), fc_scale.to(device), k, ss.to(device), off.to(device))
+    act = ops.up_swiglu_fp8(x.to(device), w_fc_q.to(device), fc_scale.to(device), k, ss.to(device), off.to(device), widen=False)
     w_fc = oracle.dequant_fp8(w_fc_q, fc_scale)
     ref_act = oracle.swiglu(oracle.scattered_experts_oracle(x, w_fc, k, se, ss, off, grouped_out=True))
     torch.testing.assert_close(act.cpu().float(), ref_act, rtol=2e-2, atol=2e-3)
-    o = ops.down_fp8(act, w_pj_q.to(device), pj_scale.to(device), ss.to(device), off.to(device))
+    o = ops.down_fp8(act, w_pj_q.to(device), pj_scale.to(device), ss.to(device), off.to(device), widen=False)
     w_pj = oracle.dequant_fp8(w_pj_q, pj_scale)
     ref_o = oracle.scattered_experts_oracle(act.cpu(), w_pj, 1, se, ss, off, grouped_in=True)
     torch.testing.assert_close(o.cpu().float(), ref_o, rtol=2e-2, atol=2e-3)
@@ -433,8 +433,8 @@ def test_fp8_tiled_layout_is_bit_identical(device, T, E, k, H, I):
     ss, off = ss.to(device), off.to(device)
     fc_t = ops.fp8_tile(w_fc_q, glu=True)
     assert torch.equal(ops.fp8_untile(fc_t, E, 2 * I, H, True).view(torch.uint8), w_fc_q.view(torch.uint8))
-    act = ops.up_swiglu_fp8(x, w_fc_q, fc_scale, k, ss, off)
-    act_t = ops.up_swiglu_fp8(x, fc_t, fc_scale, k, ss, off)
+    act = ops.up_swiglu_fp8(x, w_fc_q, fc_scale, k, ss, off, widen=False)
+    act_t = ops.up_swiglu_fp8(x, fc_t, fc_scale, k, ss, off, widen=False)
     if H >= 512:
         assert torch.equal(act, act_t)
     else:  # row-major weights with a short K take the older kernel, which sums in another order
@@ -443,8 +443,8 @@ def test_fp8_tiled_layout_is_bit_identical(device, T, E, k, H, I):
     if I % 128 == 0:
         pj_t = ops.fp8_tile(w_pj_q, glu=False)
         assert torch.equal(ops.fp8_untile(pj_t, E, H, I, False).view(torch.uint8), w_pj_q.view(torch.uint8))
-        o = ops.down_fp8(act, w_pj_q, pj_scale, ss, off)
-        o_t = ops.down_fp8(act, pj_t, pj_scale, ss, off)
+        o = ops.down_fp8(act, w_pj_q, pj_scale, ss, off, widen=False)
+        o_t = ops.down_fp8(act, pj_t, pj_scale, ss, off, widen=False)
         if I >= 512:
             assert torch.equal(o, o_t)
         else:
@@ -475,15 +475,15 @@ def test_fp8_few_rows_per_expert(device, T, E, k, H, I, skew):
     print(f"fp8 few rows T={T} E={E} k={k} H={H} I={I} max rows {counts.max().item()}", flush=True)
     xd, ssd, offd = x.to(device), ss.to(device), off.to(device)
     fc_d, fcs_d, pj_d, pjs_d = (t.to(device) for t in (w_fc_q, fc_scale, w_pj_q, pj_scale))
-    act_t = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd)
-    act_r = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd)
+    act_t = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd, widen=False)
+    act_r = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False)
     if H >= 512:
         assert torch.equal(act_t, act_r)
     ref_act = oracle.swiglu(oracle.scattered_experts_oracle(x, oracle.dequant_fp8(w_fc_q, fc_scale), k, se, ss, off,
                                                             grouped_out=True))
     torch.testing.assert_close(act_t.cpu().float(), ref_act, rtol=2e-2, atol=2e-3)
-    o_t = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd)
-    o_r = ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd)
+    o_t = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd, widen=False)
+    o_r = ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd, widen=False)
     if I >= 512:
         assert torch.equal(o_t, o_r)
     ref_o = oracle.scattered_experts_oracle(act_t.cpu(), oracle.dequant_fp8(w_pj_q, pj_scale), 1, se, ss, off,
@@ -544,10 +544,10 @@ def test_fp8_random_shapes(device, seed):
         xd, ssd, offd = x.to(device), ss.to(device), off.to(device)
         fc_d, fcs_d, pj_d, pjs_d = (t.to(device) for t in (w_fc_q, fc_scale, w_pj_q, pj_scale))
         print(f"fp8 random seed {seed} case {case}: T={T} E={E} k={k} H={H} I={I} {dtype}", flush=True)
-        act_t = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd)
-        act_r = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd)
-        o_t = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd)
-        o_r = ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd)
+        act_t = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd, widen=False)
+        act_r = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False)
+        o_t = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd, widen=False)
+        o_r = ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd, widen=False)
         if H >= 512:
             assert torch.equal(act_t, act_r), (case, "up")
         if I >= 512:
@@ -560,6 +560,78 @@ def test_fp8_random_shapes(device, seed):
                                ("down row-major", o_r, ref_o)):
             err = (got.cpu().float() - ref).abs().max().item()
             assert err <= 2e-2 * ref.abs().max().item() + 2e-3, (case, name, err)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("E,R,K,glu", [(3, 64, 256, True), (2, 40, 128, True), (5, 96, 384, False),
+                                       (2, 50, 256, False), (1, 8, 48, False), (2, 12, 80, True)])
+def test_fp8_dequant(device, dtype, E, R, K, glu):
+    """The widened weights are round(w * scale) bit for bit, from the row-major and from the tiled layout (channel
+    counts that do not fill the last unit of 16 / 32 included)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(E * 1000 + R + K)
+    w_q, scale = oracle.quantize_fp8_per_channel(torch.randn(E, R, K, generator=g) * 0.02)
+    want = (w_q.float() * scale[:, :, None]).to(dtype)
+    print(f"fp8 dequant E={E} R={R} K={K} glu={glu} {dtype}", flush=True)
+    got = ops.fp8_dequant(w_q.to(device), scale.to(device), K, glu, dtype)
+    assert got.dtype == dtype and tuple(got.shape) == (E, R, K)
+    assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
+    if K % 128 == 0:
+        tiled = ops.fp8_tile(w_q.to(device), glu)
+        got_t = ops.fp8_dequant(tiled, scale.to(device), K, glu, dtype)
+        assert torch.equal(got_t.cpu().view(torch.int16), want.view(torch.int16))
+
+
+def test_fp8_dequant_all_bit_patterns(device):
+    """Every finite e4m3fn byte value, widened with a scale of one and with one that is not a power of two."""
+    ops = _ops()
+    codes = torch.arange(256, dtype=torch.uint8)
+    finite = ~torch.isnan(codes.view(torch.float8_e4m3fn).float())
+    row = torch.where(finite, codes, torch.zeros_like(codes))
+    w_q = row.repeat(2, 16, 1).contiguous().view(torch.float8_e4m3fn)       # (2, 16, 256)
+    for sc in (1.0, 0.37):
+        scale = torch.full((2, 16), sc)
+        for dtype in (torch.bfloat16, torch.float16):
+            want = (w_q.float() * scale[:, :, None]).to(dtype)
+            for src in (w_q.to(device), ops.fp8_tile(w_q.to(device), False)):
+                got = ops.fp8_dequant(src, scale.to(device), 256, False, dtype)
+                bad = (got.cpu().view(torch.int16) != want.view(torch.int16)).nonzero()
+                assert bad.numel() == 0, (sc, dtype, src.dim(), bad[:8].tolist(),
+                                          [(float(got[tuple(b)]), float(want[tuple(b)])) for b in bad[:8]])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k,H,I", [(300, 4, 2, 256, 128), (1024, 8, 2, 512, 272), (513, 3, 1, 384, 96)])
+def test_fp8_widened_weights_for_many_rows(device, dtype, T, E, k, H, I):
+    """From 80 rows per expert on the fp8 calls widen the weights and run the tiled 16-bit kernels: same contract
+    against the oracle, the automatic choice is the widened path, and it agrees with the fp8 kernels to rounding.
+    The widened weights are rounded to the activation dtype (2^-9 relative in bf16, beside the 2^-4 of e4m3 itself),
+    which the fp8 kernels' weights are not: the absolute bound is twice that of the fp8 kernels' tests."""
+    ops = _ops()
+    atol = 4e-3 if dtype == torch.bfloat16 else 2e-3
+    g = torch.Generator().manual_seed(T + H + I)
+    se, ss, off = _routing(T, E, k, seed=T + 3)
+    x = _rand((T, H), 1.0, dtype, g)
+    w_fc_q, fc_scale = oracle.quantize_fp8_per_channel(torch.randn(E, 2 * I, H, generator=g) * 0.02)
+    w_pj_q, pj_scale = oracle.quantize_fp8_per_channel(torch.randn(E, H, I, generator=g) * 0.02)
+    xd, ssd, offd = x.to(device), ss.to(device), off.to(device)
+    fc_d, fcs_d, pj_d, pjs_d = w_fc_q.to(device), fc_scale.to(device), w_pj_q.to(device), pj_scale.to(device)
+    assert T * k >= ops.FP8_DENSE_ROWS_PER_EXPERT * E
+    print(f"fp8 widened T={T} E={E} k={k} H={H} I={I} {dtype}", flush=True)
+    act = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=True)
+    assert torch.equal(act, ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd))
+    ref_act = oracle.swiglu(oracle.scattered_experts_oracle(x, oracle.dequant_fp8(w_fc_q, fc_scale), k, se, ss, off,
+                                                           grouped_out=True))
+    torch.testing.assert_close(act.cpu().float(), ref_act, rtol=2e-2, atol=atol)
+    act_fp8 = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False)
+    torch.testing.assert_close(act.float(), act_fp8.float(), rtol=2e-2, atol=atol)
+    o = ops.down_fp8(act, pj_d, pjs_d, ssd, offd, widen=True)
+    assert torch.equal(o, ops.down_fp8(act, pj_d, pjs_d, ssd, offd))
+    ref_o = oracle.scattered_experts_oracle(act.cpu(), oracle.dequant_fp8(w_pj_q, pj_scale), 1, se, ss, off,
+                                            grouped_in=True)
+    torch.testing.assert_close(o.cpu().float(), ref_o, rtol=2e-2, atol=atol)
+    o_fp8 = ops.down_fp8(act, pj_d, pjs_d, ssd, offd, widen=False)
+    torch.testing.assert_close(o.float(), o_fp8.float(), rtol=2e-2, atol=atol)
 
 
 def test_inner_loop_probes_run(device):

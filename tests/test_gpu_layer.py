@@ -90,6 +90,15 @@ def test_layer_16bit(device, name, T):
     _check_layer(w, T, device, dict(rtol=2e-2, atol=2e-2))
 
 
+def test_layer_fp8_many_rows_per_expert(device):
+    """fp8 expert weights at a prefill-sized batch (192 rows per expert): the layer widens the weights for the call
+    and runs the tiled 16-bit kernels; same contract against the oracle as the decode batch."""
+    import dataclasses
+
+    w = dataclasses.replace(oracle.WORKLOADS["decode-fp8"], E=8, k=2, H=512, I=256, name="fp8-prefill")
+    _check_layer(w, 768, device, dict(rtol=2e-2, atol=2e-2))
+
+
 def test_layer_mixtral_shape_reduced_experts(device):
     """Mixtral-shape contraction sizes (H=4096, I=14336) with 2 experts so the CPU oracle stays small."""
     import dataclasses
