@@ -89,7 +89,7 @@ class ScatteredSwiGLUExperts(torch.autograd.Function):
         # gradient w.r.t. x: every slot's contribution in flat-slot order, then the k slots of a token summed
         dx_slots = ops.scattered_gemm(d_h, w_fc, 1, ss, off, True, False, weight_kn=True)
         # (the k slots of a token summed in slot order by the combine kernel with unit gates)
-        dx = dx_slots if k == 1 else ops.combine(dx_slots, torch.ones((T, k), dtype=x.dtype, device=x.device))
+        dx = dx_slots if k == 1 else ops.combine(dx_slots, _unit_gates(T, k, x.dtype, x.device))
         del dx_slots
 
         # weight gradients: per expert X^T dY over that expert's rows
@@ -147,7 +147,7 @@ class ScatteredExperts(torch.autograd.Function):
             # row i: d_out[orow(i)] @ w[e_i], delivered to irow(i) (kept per slot first when a token fans out to k)
             dx = ops.scattered_gemm(d_out, w, 1, ss, off, grouped_out, grouped_in, weight_kn=True)
             if not grouped_in and k > 1:
-                dx = ops.combine(dx, torch.ones((L // k, k), dtype=dx.dtype, device=dx.device))
+                dx = ops.combine(dx, _unit_gates(L // k, k, dx.dtype, dx.device))
 
         dw = None
         if need_w:
@@ -175,9 +175,22 @@ class SwitchAuxLoss(torch.autograd.Function):
 
 _ONE_EXPERT_ROWS: dict = {}
 _ONE_EXPERT_ROWS_MAX = 16
+_UNIT_GATES: dict = {}
 
 
-def _one_expert_rows(T: int, device: torch.device):
+def _unit_gates(T: int, k: int, dtype: torch.dtype, device: torch.device) -> torch.Tensor:
+    """(T, k) ones: the gates with which the combine kernel adds a token's k slots in slot order.  Read-only and
+    kept per shape like :func:`one_expert_rows` (never released; made per call beyond a few shapes)."""
+    key = (T, k, dtype, device.index)
+    hit = _UNIT_GATES.get(key)
+    if hit is None:
+        hit = torch.ones((T, k), dtype=dtype, device=device)
+        if len(_UNIT_GATES) < _ONE_EXPERT_ROWS_MAX:
+            _UNIT_GATES[key] = hit
+    return hit
+
+
+def one_expert_rows(T: int, device: torch.device):
     """(sorted_scattered_idxs, expert_offsets) of one expert that owns rows 0..T-1 in order.  Read-only and kept per
     (T, device) -- never released, so a captured graph may hold their addresses; beyond a few shapes they are made
     per call."""
@@ -215,7 +228,7 @@ class FusedRouter(torch.autograd.Function):
         if d_logits is None and d_gates is None:
             return None, None, None, None
         dl = ops.router_dlogits(logits, experts, d_gates, d_logits)
-        rows, off = _one_expert_rows(T, x.device)
+        rows, off = one_expert_rows(T, x.device)
         dx = dw = None
         if ctx.needs_input_grad[0]:
             # (T, E) @ (E, H): the gate weight transposed to (H, E) is the "(out, in)" weight of one expert

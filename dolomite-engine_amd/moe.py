@@ -29,7 +29,7 @@ import torch.nn.functional as F
 
 from . import ops
 from .activations import GLUActivation, get_activation_function, is_glu
-from .autograd import FusedRouter, ScatteredSwiGLUExperts, SwitchAuxLoss
+from .autograd import FusedRouter, ScatteredSwiGLUExperts, SwitchAuxLoss, one_expert_rows
 from .enums import Kernel
 from .kernels import is_kernel_allowed
 from .linear import ParameterizedLinear
@@ -441,8 +441,7 @@ class MoE(nn.Module):
             and hidden_states.dtype in (torch.bfloat16, torch.float16, torch.float32)
         ):
             T = hidden_states.shape[0]
-            rows = torch.arange(T, dtype=torch.int32, device=hidden_states.device)
-            offsets = torch.full((1,), T, dtype=torch.int32, device=hidden_states.device)
+            rows, offsets = one_expert_rows(T, hidden_states.device)
             w_fc, w_proj = self.c_fc_shared.weight.unsqueeze(0), self.c_proj_shared.weight.unsqueeze(0)
             if self._fused_swiglu and self._needs_grad(hidden_states):
                 return ScatteredSwiGLUExperts.apply(hidden_states, w_fc, w_proj, None, rows, offsets, 1,
