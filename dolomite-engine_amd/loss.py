@@ -13,7 +13,8 @@ def clear_aux_loss() -> None:
 
 def add_aux_loss(aux_loss: torch.Tensor | float) -> None:
     global _AUX_LOSS
-    _AUX_LOSS = _AUX_LOSS + aux_loss
+    # (the first layer's loss is taken as it is: 0 + tensor would be a kernel launch for nothing)
+    _AUX_LOSS = aux_loss if is_aux_loss_zero(_AUX_LOSS) else _AUX_LOSS + aux_loss
 
 
 def get_aux_loss() -> torch.Tensor | float:
