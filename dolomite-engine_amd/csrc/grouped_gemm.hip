@@ -1568,6 +1568,7 @@ static int dispatch_cfg(GemmArgs a, int cfg, hipStream_t s) {
     case 0: return launch_tiled<T, 256, 256, 2, 2, GLU>(a, s);
     case 1: return launch_tiled<T, 128, 128, 2, 2, GLU>(a, s);
     case 2: return launch_tiled<T, 32, 256, 1, 4, GLU>(a, s);
+    case 5: return launch_tiled<T, 32, 128, 1, 2, GLU>(a, s);
     case 4: return a.K % 32 == 0 ? launch_dma<T, 128, 128, 2, 2, GLU>(a, s) : MI_MOE_EUNSUPPORTED;
     case 7: return persistent_ok(a) ? launch_persistent<T, 256, 256, 4, 2, GLU>(a, s) : MI_MOE_EUNSUPPORTED;
     case 8:  // the persistent kernel with the tile order fixed: XCDs own contiguous ranges ...
@@ -1587,6 +1588,7 @@ static int dispatch_cfg_f32(GemmArgs a, int cfg, hipStream_t s) {
     case 0: return launch_tiled<float, 256, 256, 2, 2, GLU>(a, s);
     case 1: return launch_tiled<float, 128, 128, 2, 2, GLU>(a, s);
     case 2: return launch_tiled<float, 32, 256, 1, 4, GLU>(a, s);
+    case 5: return launch_tiled<float, 32, 128, 1, 2, GLU>(a, s);
     default: return MI_MOE_EUNSUPPORTED;
   }
 }
@@ -1608,7 +1610,11 @@ static int pick_cfg(const GemmArgs& a) {
   if (avg >= 192 && persistent_ok(a)) return 7;
   if (avg >= 512) return 0;
   if (avg >= 48) return a.K % 32 == 0 ? 4 : 1;
-  return 2;
+  // A few rows per expert: every weight byte is used once and the kernel is a weight stream, which wants many
+  // workgroups.  Measured at 8 - 256 tokens (kernel times, up / down projection): hidden 1536, 40 experts -- 32 x 256
+  // tiles 29 - 31 / 13.5 - 17 us, 32 x 128 tiles 23 - 27 / 12 - 17 us, DMA-staged 128 x 128 tiles 28 - 30 / 13 - 16 us;
+  // hidden 1024, 32 experts -- 20 - 22 / 12 - 15, 16 - 21 / 9 - 13, 15 - 16 / 9 - 11 us.
+  return (a.K % 32 == 0 && a.K <= 1024) ? 4 : 5;
 }
 
 // cfg < 0 picks a matrix-core kernel from the shape.  Nothing drops to the one-thread-per-output kernel on its own:
@@ -1643,7 +1649,7 @@ static int run_gemm(GemmArgs a, int dtype, bool glu, int cfg, int in_rows_bound,
   if (dtype == MI_MOE_F32) {
     if (cfg < 0) {
       const long avg = a.E > 0 ? (long)a.L / a.E : a.L;
-      cfg = avg >= 512 ? 0 : (avg >= 48 ? 1 : 2);
+      cfg = avg >= 512 ? 0 : (avg >= 48 ? 1 : 5);
     }
     return glu ? dispatch_cfg_f32<true>(a, cfg, s) : dispatch_cfg_f32<false>(a, cfg, s);
   }

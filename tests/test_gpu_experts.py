@@ -55,7 +55,7 @@ CASES = [
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,E,k,K,N", CASES)
 @pytest.mark.parametrize("mode", ["scatter2group", "group2scatter", "scatter2scatter", "group2group"])
-@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4, 7, 8, 9])
+@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4, 5, 7, 8, 9])
 def test_scattered_gemm(device, dtype, T, E, k, K, N, mode, cfg):
     if dtype == torch.float32 and cfg in (4, 7, 8, 9):
         pytest.skip("the DMA-staged configurations are 16-bit only")
@@ -106,7 +106,7 @@ def test_scattered_gemm_weight_kn(device, dtype, T, E, k, K, N, mode):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,E,k,H,I", [(15, 8, 8, 32, 128), (512, 8, 2, 256, 512), (333, 5, 2, 136, 100),
                                        (2048, 4, 2, 512, 256), (64, 64, 6, 256, 128)])
-@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4, 7, 8, 9])
+@pytest.mark.parametrize("cfg", [-1, 0, 1, 2, 3, 4, 5, 7, 8, 9])
 def test_up_swiglu(device, dtype, T, E, k, H, I, cfg):
     if dtype == torch.float32 and cfg in (4, 7, 8, 9):
         pytest.skip("the DMA-staged configurations are 16-bit only")
@@ -140,7 +140,7 @@ def test_gemm_identity_weights_permutes_rows(device):
     assert torch.equal(out2.cpu(), x.repeat_interleave(k, dim=0))
 
 
-@pytest.mark.parametrize("cfg", [2, 3, 4, 7, 9])
+@pytest.mark.parametrize("cfg", [2, 3, 4, 5, 7, 9])
 def test_gemm_bf16_rounding_is_nearest_even(device, cfg):
     """The final fp32 -> bf16 rounding is round-to-nearest-even, bit for bit (ties, carries into the
     exponent, overflow to inf, NaN): out = a + b where the fp32 sum is exact, so the only rounding in the
@@ -186,7 +186,7 @@ def test_gemm_empty_experts_and_single_expert(device):
     se, ss, off = oracle.sort_bin(sel, E)
     x = _rand((T, K), 1.0, torch.bfloat16, g)
     w = _rand((E, N, K), 0.05, torch.bfloat16, g)
-    for cfg in (0, 1, 2, 3, 4, 7, 8, 9):
+    for cfg in (0, 1, 2, 3, 4, 5, 7, 8, 9):
         out = ops.scattered_gemm(x.to(device), w.to(device), k, ss.to(device), off.to(device), False, False, cfg=cfg)
         ref = x.float() @ w[9].float().t()
         torch.testing.assert_close(out.cpu().float(), ref, rtol=2e-2, atol=2e-2)
