@@ -1613,8 +1613,10 @@ static int pick_cfg(const GemmArgs& a) {
   // A few rows per expert: every weight byte is used once and the kernel is a weight stream, which wants many
   // workgroups.  Measured at 8 - 256 tokens (kernel times, up / down projection): hidden 1536, 40 experts -- 32 x 256
   // tiles 29 - 31 / 13.5 - 17 us, 32 x 128 tiles 23 - 27 / 12 - 17 us, DMA-staged 128 x 128 tiles 28 - 30 / 13 - 16 us;
-  // hidden 1024, 32 experts -- 20 - 22 / 12 - 15, 16 - 21 / 9 - 13, 15 - 16 / 9 - 11 us.
-  return (a.K % 32 == 0 && a.K <= 1024) ? 4 : 5;
+  // hidden 1024, 32 experts -- 20 - 22 / 12 - 15, 16 - 21 / 9 - 13, 15 - 16 / 9 - 11 us.  A very long contraction
+  // (the down-projection of an intermediate size of 14336: 226 against 188 us at 64 tokens) wants the deeper ring of
+  // the DMA-staged kernel too.
+  return (a.K % 32 == 0 && (a.K <= 1024 || a.K >= 8192)) ? 4 : 5;
 }
 
 // cfg < 0 picks a matrix-core kernel from the shape.  Nothing drops to the one-thread-per-output kernel on its own:
