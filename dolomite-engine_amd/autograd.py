@@ -185,9 +185,15 @@ def _unit_gates(T: int, k: int, dtype: torch.dtype, device: torch.device) -> tor
     hit = _UNIT_GATES.get(key)
     if hit is None:
         hit = torch.ones((T, k), dtype=dtype, device=device)
-        if len(_UNIT_GATES) < _ONE_EXPERT_ROWS_MAX:
+        if len(_UNIT_GATES) < _ONE_EXPERT_ROWS_MAX and not _capturing():
             _UNIT_GATES[key] = hit
     return hit
+
+
+def _capturing() -> bool:
+    """A tensor filled while a graph is being captured holds its values only once the graph has run: such tensors
+    are not kept for later calls."""
+    return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
 
 
 def one_expert_rows(T: int, device: torch.device):
@@ -199,7 +205,7 @@ def one_expert_rows(T: int, device: torch.device):
     if hit is not None:
         return hit
     made = (torch.arange(T, dtype=torch.int32, device=device), torch.full((1,), T, dtype=torch.int32, device=device))
-    if len(_ONE_EXPERT_ROWS) < _ONE_EXPERT_ROWS_MAX:
+    if len(_ONE_EXPERT_ROWS) < _ONE_EXPERT_ROWS_MAX and not _capturing():
         _ONE_EXPERT_ROWS[key] = made
     return made
 
