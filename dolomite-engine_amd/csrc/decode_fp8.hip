@@ -458,13 +458,28 @@ static int dispatch_decode(const DecodeArgs& a, hipStream_t s) {
   return launch_decode<T, GLU, 1>(a, s);
 }
 
-static int run_decode(DecodeArgs a, int dtype, bool glu, hipStream_t s) {
+// grouped_gemm.hip: the same product on the register-staged tile kernels, fp8 bytes widened on their way into LDS
+int mi_gemm_fp8_tiled(const void* in, const void* wq, const float* scale, void* out, const int32_t* sorted_scattered,
+                      const int32_t* expert_offsets, int L, int K, int N, int E, int kdiv, int gather, int scatter,
+                      int glu, int w_tiled, int dtype, hipStream_t s);
+
+// Rows per expert (on average) from which the tile kernels take over: the streaming kernels read an expert's
+// weights once per 16 of its rows, a tile kernel once per row tile.  Measured on 64 experts of 2 x 1408 x 4096 and
+// 4096 x 1408 weights, top-6, both projections: 12 rows per expert 224 us streaming / 266 us tiles, 18 rows 339 / 273,
+// 48 rows 762 / 383, 96 rows 1448 / 410.
+#define FP8_TILED_MIN_ROWS 16
+
+static int run_decode(DecodeArgs a, int dtype, bool glu, hipStream_t s, int form) {
   if (a.L < 0 || a.K < 1 || a.N < 1 || a.E < 1 || a.kdiv < 1) return MI_MOE_ESHAPE;
   if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
   if (a.L == 0) return MI_MOE_OK;
   if (!a.in || !a.wq || !a.scale || !a.out || !a.expert_offsets) return MI_MOE_ENULL;
   if ((a.gather || a.scatter) && !a.sorted_scattered) return MI_MOE_ENULL;
   if (a.K % 16 != 0 || a.N % 4 != 0) return MI_MOE_EUNSUPPORTED;
+  // form: 0 by the batch, 1 the streaming kernels, 2 the tile kernels
+  if (form == 2 || (form == 0 && (long)a.L >= (long)FP8_TILED_MIN_ROWS * a.E))
+    return mi_gemm_fp8_tiled(a.in, a.wq, a.scale, a.out, a.sorted_scattered, a.expert_offsets, a.L, a.K, a.N, a.E,
+                             a.kdiv, a.gather, a.scatter, glu ? 1 : 0, a.tiled ? 1 : 0, dtype, s);
   if (!mi_aligned(a.in, 16) || !mi_aligned(a.wq, 16) || !mi_aligned(a.scale, 16) || !mi_aligned(a.out, 8))
     return MI_MOE_EALIGN;
   if (dtype == MI_MOE_BF16) return glu ? dispatch_decode<bf16_t, true>(a, s) : dispatch_decode<bf16_t, false>(a, s);
@@ -477,26 +492,46 @@ extern "C" size_t mi_moe_fp8_tiled_bytes(int E, int N, int K, int glu) {
   return (size_t)E * mi_ceil_div(N, chw) * (size_t)(K / 128) * 4096;
 }
 
-extern "C" int mi_moe_up_swiglu_fp8(const void* x, const void* w_fc_q, const float* w_fc_scale, void* act_out,
-                                    const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int H,
-                                    int I, int E, int k, int dtype, int w_tiled, mi_moe_stream_t stream) {
+// cfg: -1 picks by the batch (tile kernels from FP8_TILED_MIN_ROWS rows per expert on average), 0 the streaming
+// kernels, 1 the tile kernels
+static int fp8_form(int cfg) { return cfg < 0 ? 0 : (cfg == 0 ? 1 : 2); }
+
+extern "C" int mi_moe_up_swiglu_fp8_cfg(const void* x, const void* w_fc_q, const float* w_fc_scale, void* act_out,
+                                        const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int H,
+                                        int I, int E, int k, int dtype, int w_tiled, int cfg, mi_moe_stream_t stream) {
+  if (cfg < -1 || cfg > 1) return MI_MOE_EUNSUPPORTED;
   DecodeArgs a;
   a.in = x; a.wq = static_cast<const uint8_t*>(w_fc_q); a.scale = w_fc_scale; a.out = act_out;
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = H; a.N = I; a.E = E; a.kdiv = k; a.gather = 1; a.scatter = 0; a.groups_per_expert = 0;
   a.tiled = w_tiled != 0;
-  return run_decode(a, dtype, true, static_cast<hipStream_t>(stream));
+  return run_decode(a, dtype, true, static_cast<hipStream_t>(stream), fp8_form(cfg));
 }
 
-extern "C" int mi_moe_down_fp8(const void* act, const void* w_proj_q, const float* w_proj_scale, void* o_out,
-                               const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
-                               int E, int dtype, int w_tiled, mi_moe_stream_t stream) {
+extern "C" int mi_moe_up_swiglu_fp8(const void* x, const void* w_fc_q, const float* w_fc_scale, void* act_out,
+                                    const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int H,
+                                    int I, int E, int k, int dtype, int w_tiled, mi_moe_stream_t stream) {
+  return mi_moe_up_swiglu_fp8_cfg(x, w_fc_q, w_fc_scale, act_out, sorted_scattered, expert_offsets, L, H, I, E, k, dtype,
+                                  w_tiled, -1, stream);
+}
+
+extern "C" int mi_moe_down_fp8_cfg(const void* act, const void* w_proj_q, const float* w_proj_scale, void* o_out,
+                                   const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
+                                   int E, int dtype, int w_tiled, int cfg, mi_moe_stream_t stream) {
+  if (cfg < -1 || cfg > 1) return MI_MOE_EUNSUPPORTED;
   DecodeArgs a;
   a.in = act; a.wq = static_cast<const uint8_t*>(w_proj_q); a.scale = w_proj_scale; a.out = o_out;
   a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
   a.L = L; a.K = I; a.N = H; a.E = E; a.kdiv = 1; a.gather = 0; a.scatter = 1; a.groups_per_expert = 0;
   a.tiled = w_tiled != 0;
-  return run_decode(a, dtype, false, static_cast<hipStream_t>(stream));
+  return run_decode(a, dtype, false, static_cast<hipStream_t>(stream), fp8_form(cfg));
+}
+
+extern "C" int mi_moe_down_fp8(const void* act, const void* w_proj_q, const float* w_proj_scale, void* o_out,
+                               const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
+                               int E, int dtype, int w_tiled, mi_moe_stream_t stream) {
+  return mi_moe_down_fp8_cfg(act, w_proj_q, w_proj_scale, o_out, sorted_scattered, expert_offsets, L, I, H, E, dtype,
+                             w_tiled, -1, stream);
 }
 
 // ---- fp8 weights -> 16-bit weights with the channel scale folded in ----------------------------------------------

@@ -97,6 +97,36 @@ struct GemmArgs {
   void* ws;     // persistent kernel: workspace for splitting the last round of tiles along K (or null)
   void* pre;    // persistent SwiGLU kernel: (L, 2N) pre-activation output next to the activation (or null)
   int out_nt;   // persistent kernel: store the output non-temporal (set in run_gemm)
+  // fp8 weights (register-staged kernel, W8 form): w holds e4m3fn bytes, row-major (E, rows, K) or in the streamed-tile
+  // layout of decode_fp8.hip; wscale (E, rows) fp32 is applied to the accumulators in the epilogue
+  const float* wscale;
+  int w_tiled;
+};
+
+// 8 fp8 e4m3fn values (two dwords) -> 8 values of a 16-bit type (exact: e4m3 fits in either)
+template <typename T> struct Widen8;
+template <> struct Widen8<bf16_t> {
+  static __device__ __forceinline__ u32x4 run(uint32_t lo, uint32_t hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const bf16x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
+    const bf16x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+    const bf16x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
+    const bf16x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+    return (u32x4){__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1), __builtin_bit_cast(uint32_t, p2),
+                   __builtin_bit_cast(uint32_t, p3)};
+  }
+};
+template <> struct Widen8<f16_t> {
+  static __device__ __forceinline__ u32x4 run(uint32_t lo, uint32_t hi) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const f32x2 p0 = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(lo, true);
+    const f32x2 p2 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), p3 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+    return (u32x4){pack2<f16_t>(p0[0], p0[1]), pack2<f16_t>(p1[0], p1[1]), pack2<f16_t>(p2[0], p2[1]),
+                   pack2<f16_t>(p3[0], p3[1])};
+  }
+};
+template <> struct Widen8<float> {  // (not used: fp32 activations have no fp8 form)
+  static __device__ __forceinline__ u32x4 run(uint32_t, uint32_t) { return (u32x4){0u, 0u, 0u, 0u}; }
 };
 
 
@@ -173,8 +203,13 @@ __device__ __forceinline__ bool decode_tile(const int32_t* __restrict__ off, int
 #define SG_DS_RD 0x100
 #define SG_DS_WR 0x200
 
-template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool KTAIL>
+// W8: the weights are fp8 e4m3fn bytes with one fp32 scale per weight row (a.wscale); a thread fetches the 8 bytes
+// of its chunk and widens them on their way into LDS, the scale meets the accumulators in the epilogue.  For batches
+// between decode (decode_fp8.hip streams an expert's weights once per 16 rows) and the sizes where widening all
+// weights first pays (mi_moe_fp8_dequant).
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool KTAIL, bool W8 = false>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
+  static_assert(!W8 || sizeof(T) == 2, "fp8 weights go with 16-bit activations");
   constexpr int CE = 16 / sizeof(T);        // elements per 16-byte chunk (8 for the 16-bit types, 4 for fp32)
   constexpr int BK = 8 * CE;                // K tile: 128 bytes per row
   constexpr int NT = WM * WN * 64;
@@ -212,7 +247,16 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
   const int r0 = tid / CPR;  // first tile row of this thread
   constexpr int WROWS_MUL = GLU ? 2 : 1;
   const T* __restrict__ xbase = static_cast<const T*>(a.in);
-  const T* __restrict__ wbase = static_cast<const T*>(a.w) + (size_t)expert * WROWS_MUL * a.N * a.K;
+  const T* __restrict__ wbase = static_cast<const T*>(a.w) + (W8 ? 0 : (size_t)expert * WROWS_MUL * a.N * a.K);
+  // W8: byte address of the expert's weights; woff[j] is a byte offset (row-major: of the row's chunk c; tiled: of
+  // the row inside stage 0 of its unit) and wfx[j] the row's slot swizzle in the tiled layout
+  const uint8_t* __restrict__ wbase8 = nullptr;
+  if constexpr (W8) {
+    const size_t expert_bytes =
+        a.w_tiled ? (size_t)mi_ceil_div_dev(a.N, GLU ? 16 : 32) * (size_t)(a.K >> 7) * 4096 : (size_t)WROWS_MUL * a.N * a.K;
+    wbase8 = static_cast<const uint8_t*>(a.w) + (size_t)expert * expert_bytes;
+  }
+  int wfx[WCH];
 
   uint32_t xoff[XCH], woff[WCH];
 #pragma unroll
@@ -234,6 +278,16 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
     }
     if (col > a.N - 1) col = a.N - 1;  // column tail re-reads the last weight row; never stored
     woff[j] = (uint32_t)(half * a.N + col) * (uint32_t)a.K + c * CE;
+    wfx[j] = 0;
+    if constexpr (W8) {
+      if (a.w_tiled) {
+        // unit u = 16 up + 16 gate channels (GLU) or 32 channels; row t of the unit's 32-row stage image
+        const int u = GLU ? col >> 4 : col >> 5;
+        const int t = GLU ? (col & 15) + 16 * half : (col & 31);
+        woff[j] = (uint32_t)u * (uint32_t)(a.K >> 7) * 4096u + (uint32_t)t * 128u;
+        wfx[j] = ((t >> 1) & 1) | (((t >> 2) & 1) << 2);
+      }
+    }
   }
 
   // LDS tile layout: row r holds its eight 16-byte chunks at slots  chunk ^ swz(r),
@@ -245,7 +299,15 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
   const int st_w = BM * BK + (r0 * CPR + sw_c) * CE;    // ... inside the W tile (after the X tile)
 
   u32x4 xreg[XCH], wreg[WCH];
+  u32x2 wraw[W8 ? WCH : 1];  // W8: the chunk's 8 bytes as loaded (widened when they go to LDS)
   const int nk = (a.K + BK - 1) / BK;
+  // W8: byte offset of this thread's 8-byte chunk of the K tile that starts at k0 (tiled: K % 128 == 0, so every
+  // chunk exists and kc = k0 + 8 c < K)
+  auto w8_at = [&](int j, int k0) -> uint32_t {
+    if (!a.w_tiled) return woff[j] + (uint32_t)k0;
+    const int kc = k0 + c * CE;
+    return woff[j] + (uint32_t)(kc >> 7) * 4096u + (uint32_t)((((kc & 127) >> 4) ^ wfx[j]) << 4) + (uint32_t)(kc & 8);
+  };
 
   auto load_global = [&](int kt) {
     int k0 = kt * BK;
@@ -260,14 +322,23 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
       }
 #pragma unroll
       for (int j = 0; j < WCH; ++j) {
-        u32x4 v = *reinterpret_cast<const u32x4*>(wbase + woff[j] + koff);
-        wreg[j] = kvalid ? v : (u32x4){0u, 0u, 0u, 0u};
+        if constexpr (W8) {
+          // (a partial K tile only exists with row-major weights: the tiled layout has whole 128-wide stages)
+          const u32x2 v = *reinterpret_cast<const u32x2*>(wbase8 + woff[j] + koff);
+          wraw[j] = kvalid ? v : (u32x2){0u, 0u};
+        } else {
+          u32x4 v = *reinterpret_cast<const u32x4*>(wbase + woff[j] + koff);
+          wreg[j] = kvalid ? v : (u32x4){0u, 0u, 0u, 0u};
+        }
       }
     } else {
 #pragma unroll
       for (int j = 0; j < XCH; ++j) xreg[j] = *reinterpret_cast<const u32x4*>(xbase + xoff[j] + k0);
 #pragma unroll
-      for (int j = 0; j < WCH; ++j) wreg[j] = *reinterpret_cast<const u32x4*>(wbase + woff[j] + k0);
+      for (int j = 0; j < WCH; ++j) {
+        if constexpr (W8) wraw[j] = *reinterpret_cast<const u32x2*>(wbase8 + w8_at(j, k0));
+        else wreg[j] = *reinterpret_cast<const u32x4*>(wbase + woff[j] + k0);
+      }
     }
   };
   // chunk writes [first, first + count) of this thread's NWR chunks (X chunks first, then W chunks)
@@ -278,6 +349,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
       if (j < first || j >= first + count) continue;
       if (j < XCH)
         *reinterpret_cast<u32x4*>(s + st_x + j * RS * BK) = xreg[j];
+      else if constexpr (W8)
+        *reinterpret_cast<u32x4*>(s + st_w + (j - XCH) * RS * BK) = Widen8<T>::run(wraw[j - XCH][0], wraw[j - XCH][1]);
       else
         *reinterpret_cast<u32x4*>(s + st_w + (j - XCH) * RS * BK) = wreg[j - XCH];
     }
@@ -413,14 +486,25 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GemmArgs a) {
         const int col = col0 + g * 8;
         if (col >= a.N) continue;
         float v[4];
+        f32x4 su = {1.f, 1.f, 1.f, 1.f}, sg = {1.f, 1.f, 1.f, 1.f};
+        if constexpr (W8) {  // (N % 4 == 0 and col % 4 == 0: the four columns exist together)
+          const float* sc = a.wscale + (size_t)expert * WROWS_MUL * a.N + col;
+          su = *reinterpret_cast<const f32x4*>(sc);
+          if (GLU) sg = *reinterpret_cast<const f32x4*>(sc + a.N);
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           if (GLU) {
             float up = acc[nb][mb][g * 4 + i];
             float gt = acc[nb + NB / 2][mb][g * 4 + i];
+            if constexpr (W8) {
+              up *= su[i];
+              gt *= sg[i];
+            }
             v[i] = up * silu_f32(gt);
           } else {
             v[i] = acc[nb][mb][g * 4 + i];
+            if constexpr (W8) v[i] *= su[i];
           }
         }
         if constexpr (sizeof(T) == 4) {
@@ -1451,11 +1535,11 @@ __global__ __launch_bounds__(256) void grouped_gemm_naive_kernel(GemmArgs a) {
 
 // ---- host side ------------------------------------------------------------------------------------
 
-template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool KTAIL>
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU, bool KTAIL, bool W8 = false>
 static int launch_tiled_k(GemmArgs a, hipStream_t s) {
   constexpr int BN = GLU ? BNW / 2 : BNW;
   constexpr size_t lds = 2ull * (BM + BNW) * 128;  // two stages of 128-byte rows
-  auto kern = grouped_gemm_kernel<T, BM, BNW, WM, WN, GLU, KTAIL>;
+  auto kern = grouped_gemm_kernel<T, BM, BNW, WM, WN, GLU, KTAIL, W8>;
   if (lds > 64 * 1024) {
     static std::atomic<uint64_t> lds_ok{0};
     const int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), (int)lds, lds_ok);
@@ -1474,6 +1558,13 @@ template <typename T, int BM, int BNW, int WM, int WN, bool GLU>
 static int launch_tiled(GemmArgs a, hipStream_t s) {
   if (a.K % (128 / (int)sizeof(T)) == 0) return launch_tiled_k<T, BM, BNW, WM, WN, GLU, false>(a, s);
   return launch_tiled_k<T, BM, BNW, WM, WN, GLU, true>(a, s);
+}
+
+// fp8 weights (K tiles of 64 values: 64 bytes of a weight row)
+template <typename T, int BM, int BNW, int WM, int WN, bool GLU>
+static int launch_tiled_w8(GemmArgs a, hipStream_t s) {
+  if (a.K % 64 == 0) return launch_tiled_k<T, BM, BNW, WM, WN, GLU, false, true>(a, s);
+  return launch_tiled_k<T, BM, BNW, WM, WN, GLU, true, true>(a, s);
 }
 
 template <typename T, int BM, int BNW, int WM, int WN, bool GLU>
@@ -1525,6 +1616,40 @@ static int launch_persistent(GemmArgs a, hipStream_t s) {
   hipLaunchKernelGGL((grouped_gemm_split_finish_kernel<T, BM, BNW, WM, WN, GLU>), dim3(8u * (unsigned)((nslot + 1) / 2)),
                      dim3(NW * 64), 0, s, a, nslot);
   return mi_launch_status();
+}
+
+// fp8 expert weights on the register-staged tiles: out[orow(i)] = scale[e_i] * (in[irow(i)] @ Wq[e_i]^T), with SwiGLU
+// over the [up ; gate] halves when glu.  Called by decode_fp8.hip for batches beyond a few rows per expert (the
+// streaming kernels there read an expert's weights once per 16 of its rows).  Shapes: K % 16 == 0, N % 4 == 0,
+// w_tiled only with K % 128 == 0; MI_MOE_EUNSUPPORTED otherwise.
+template <typename T, bool GLU>
+static int dispatch_w8(const GemmArgs& a, hipStream_t s) {
+  const long avg = a.E > 0 ? (long)a.L / a.E : a.L;
+  if (avg >= 512) return launch_tiled_w8<T, 256, 256, 2, 2, GLU>(a, s);
+  if (avg >= 48) return launch_tiled_w8<T, 128, 128, 2, 2, GLU>(a, s);
+  return launch_tiled_w8<T, 32, 128, 1, 2, GLU>(a, s);
+}
+
+int mi_gemm_fp8_tiled(const void* in, const void* wq, const float* scale, void* out, const int32_t* sorted_scattered,
+                      const int32_t* expert_offsets, int L, int K, int N, int E, int kdiv, int gather, int scatter,
+                      int glu, int w_tiled, int dtype, hipStream_t s) {
+  if (dtype != MI_MOE_BF16 && dtype != MI_MOE_F16) return MI_MOE_EDTYPE;
+  if (L == 0) return MI_MOE_OK;
+  if (K % 16 != 0 || N % 4 != 0 || (w_tiled && K % 128 != 0)) return MI_MOE_EUNSUPPORTED;
+  // 32-bit element offsets into the activations, 32-bit byte offsets inside one expert's weights
+  const double in_rows = gather ? (double)L / (kdiv > 0 ? kdiv : 1) : (double)L;
+  if (in_rows * K >= 2147483648.0) return MI_MOE_EUNSUPPORTED;
+  const double wrows = w_tiled ? (double)mi_ceil_div(N, glu ? 16 : 32) * 32 : (double)(glu ? 2 : 1) * N;
+  if (wrows * K >= 2147483648.0) return MI_MOE_EUNSUPPORTED;
+  if (!mi_aligned(in, 16) || !mi_aligned(wq, 16) || !mi_aligned(scale, 16) || !mi_aligned(out, 8)) return MI_MOE_EALIGN;
+  GemmArgs a;
+  a.in = in; a.w = wq; a.out = out;
+  a.sorted_scattered = sorted_scattered; a.expert_offsets = expert_offsets;
+  a.L = L; a.K = K; a.N = N; a.E = E; a.kdiv = kdiv > 0 ? kdiv : 1; a.kshift = -1; a.n_tiles = 0;
+  a.gather = gather; a.scatter = scatter; a.remap = 1; a.ws = nullptr; a.pre = nullptr; a.out_nt = 0;
+  a.wscale = scale; a.w_tiled = w_tiled;
+  if (dtype == MI_MOE_BF16) return glu ? dispatch_w8<bf16_t, true>(a, s) : dispatch_w8<bf16_t, false>(a, s);
+  return glu ? dispatch_w8<f16_t, true>(a, s) : dispatch_w8<f16_t, false>(a, s);
 }
 
 // workspace of the persistent kernel: one fp32 partial tile per workgroup of the largest grid

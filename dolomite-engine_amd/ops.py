@@ -792,10 +792,12 @@ def fp8_untile(tiled: torch.Tensor, E: int, out_rows: int, K: int, glu: bool) ->
     return w.contiguous().view(torch.float8_e4m3fn)
 
 
-# Average rows per expert from which the fp8 calls widen the weights for the call and run the tiled 16-bit kernels
-# instead: the fp8 kernels stream an expert's weights once per 16 of its rows (right for decode, linear in the
-# batch beyond), the widening is one pass over the weights whatever the batch.
-FP8_DENSE_ROWS_PER_EXPERT = 80
+# Average rows per expert from which the fp8 calls widen the weights for the call and run the persistent 16-bit
+# kernels instead of the library's own fp8 kernels (streaming for a few rows per expert, tiles that widen the bytes
+# on their way into LDS beyond): the widening is one pass over all weights whatever the batch, and the persistent
+# kernel is the faster GEMM.  Measured on the decode workload's shape (both projections): 384 rows per expert 1.34 ms
+# on the fp8 tiles / 1.58 ms widened, 768 rows 2.27 / 2.23 ms, 1536 rows 4.16 / 3.55 ms.
+FP8_DENSE_ROWS_PER_EXPERT = 768
 
 
 def fp8_dequant(w_q: torch.Tensor, scale: torch.Tensor, in_features: int, glu: bool, dtype: torch.dtype) -> torch.Tensor:
@@ -827,11 +829,13 @@ def fp8_dequant(w_q: torch.Tensor, scale: torch.Tensor, in_features: int, glu: b
 
 def up_swiglu_fp8(x: torch.Tensor, w_fc_q: torch.Tensor, w_fc_scale: torch.Tensor, k: int,
                   sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor,
-                  widen: bool | None = None) -> torch.Tensor:
+                  widen: bool | None = None, cfg: int = -1) -> torch.Tensor:
     """As up_swiglu with e4m3fn weights and fp32 per-output-channel scales (E, 2I).  The weights are either
     row-major (E, 2I, H) or, as a flat tensor, in the layout of :func:`fp8_tile` (``glu=True``).  From
     FP8_DENSE_ROWS_PER_EXPERT rows per expert on average the weights are widened for the call and
-    :func:`up_swiglu` runs on the copy (``widen``: True / False force either way)."""
+    :func:`up_swiglu` runs on the copy (``widen``: True / False force either way).  Below that the library picks
+    between its streaming kernels (decode: a few rows per expert) and the tile kernels that widen the fp8 bytes on
+    their way into LDS (``cfg``: 0 / 1 force either, -1 picks by the batch)."""
     _dev(x, w_fc_q, w_fc_scale, sorted_scattered_idxs, expert_offsets)
     _no_grad(x)
     if w_fc_q.dtype != torch.float8_e4m3fn:
@@ -857,17 +861,17 @@ def up_swiglu_fp8(x: torch.Tensor, w_fc_q: torch.Tensor, w_fc_scale: torch.Tenso
         return up_swiglu(x, fp8_dequant(w_fc_q, scale, H, True, x.dtype), k, ss, off)
     act = torch.empty((L, I2 // 2), dtype=x.dtype, device=x.device)
     with _stage("up_swiglu_fp8"):
-        check(lib.mi_moe_up_swiglu_fp8(_ptr(x), _ptr(w_fc_q), _ptr(scale), _ptr(act), _ptr(ss), _ptr(off), L, H,
-                                      I2 // 2, E, k, _code(x.dtype), int(tiled), _stream()))
+        check(lib.mi_moe_up_swiglu_fp8_cfg(_ptr(x), _ptr(w_fc_q), _ptr(scale), _ptr(act), _ptr(ss), _ptr(off), L, H,
+                                          I2 // 2, E, k, _code(x.dtype), int(tiled), int(cfg), _stream()))
     return act
 
 
 def down_fp8(act: torch.Tensor, w_proj_q: torch.Tensor, w_proj_scale: torch.Tensor,
              sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor,
-             widen: bool | None = None) -> torch.Tensor:
+             widen: bool | None = None, cfg: int = -1) -> torch.Tensor:
     """Down-projection with e4m3fn weights, row-major (E, H, I) or tiled (:func:`fp8_tile`, ``glu=False``):
     act (L, I) grouped -> (L, H) in flat-slot order (widened weights from FP8_DENSE_ROWS_PER_EXPERT rows per expert
-    on, as in :func:`up_swiglu_fp8`)."""
+    on, ``cfg`` below that, as in :func:`up_swiglu_fp8`)."""
     _dev(act, w_proj_q, w_proj_scale, sorted_scattered_idxs, expert_offsets)
     _no_grad(act)
     if w_proj_q.dtype != torch.float8_e4m3fn:
@@ -892,6 +896,6 @@ def down_fp8(act: torch.Tensor, w_proj_q: torch.Tensor, w_proj_scale: torch.Tens
         return scattered_gemm(act, fp8_dequant(w_proj_q, scale, I, False, act.dtype), 1, ss, off, True, False)
     o = torch.empty((L, H), dtype=act.dtype, device=act.device)
     with _stage("down_fp8"):
-        check(lib.mi_moe_down_fp8(_ptr(act), _ptr(w_proj_q), _ptr(scale), _ptr(o), _ptr(ss), _ptr(off), L, I, H,
-                                 E, _code(act.dtype), int(tiled), _stream()))
+        check(lib.mi_moe_down_fp8_cfg(_ptr(act), _ptr(w_proj_q), _ptr(scale), _ptr(o), _ptr(ss), _ptr(off), L, I, H,
+                                     E, _code(act.dtype), int(tiled), int(cfg), _stream()))
     return o

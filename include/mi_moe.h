@@ -380,6 +380,16 @@ int mi_moe_up_swiglu_fp8(const void* x, const void* w_fc_q, const float* w_fc_sc
 int mi_moe_down_fp8(const void* act, const void* w_proj_q, const float* w_proj_scale, void* o_out,
                     const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
                     int E, int dtype, int w_tiled, mi_moe_stream_t stream);
+/* The same two calls with the kernel family chosen by the caller: cfg -1 picks by the batch (what the calls above
+ * do), 0 the streaming kernels (an expert's weights are read once per 16 of its rows: decode), 1 the tile kernels of
+ * the grouped GEMM with the fp8 bytes widened on their way into LDS (an expert's weights are read once per row tile:
+ * from a few dozen rows per expert on). */
+int mi_moe_up_swiglu_fp8_cfg(const void* x, const void* w_fc_q, const float* w_fc_scale, void* act_out,
+                             const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int H, int I,
+                             int E, int k, int dtype, int w_tiled, int cfg, mi_moe_stream_t stream);
+int mi_moe_down_fp8_cfg(const void* act, const void* w_proj_q, const float* w_proj_scale, void* o_out,
+                        const int32_t* sorted_scattered, const int32_t* expert_offsets, int L, int I, int H,
+                        int E, int dtype, int w_tiled, int cfg, mi_moe_stream_t stream);
 /* The same weights widened to `dtype` with the channel scale folded in: w_out (E, out, in) -- (E, 2 * out, in), up
  * rows first, with glu -- = round(w * scale[:, None]), from either layout.  For batches with many rows per expert,
  * where the two calls above (which stream an expert's weights once per 16 of its rows) lose to the tiled 16-bit

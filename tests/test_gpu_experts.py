@@ -408,11 +408,11 @@ def test_fp8_up_down(device, dtype, T, E, k, H, I):
     w_fc_q, fc_scale = oracle.quantize_fp8_per_channel(torch.randn(E, 2 * I, H, generator=g) * 0.02)
     w_pj_q, pj_scale = oracle.quantize_fp8_per_channel(torch.randn(E, H, I, generator=g) * 0.02)
     print(f"fp8 T={T} E={E} k={k} H={H} I={I} {dtype}", flush=True)
-    act = ops.up_swiglu_fp8(x.to(device), w_fc_q.to(device), fc_scale.to(device), k, ss.to(device), off.to(device), widen=False)
+    act = ops.up_swiglu_fp8(x.to(device), w_fc_q.to(device), fc_scale.to(device), k, ss.to(device), off.to(device), widen=False, cfg=0)
     w_fc = oracle.dequant_fp8(w_fc_q, fc_scale)
     ref_act = oracle.swiglu(oracle.scattered_experts_oracle(x, w_fc, k, se, ss, off, grouped_out=True))
     torch.testing.assert_close(act.cpu().float(), ref_act, rtol=2e-2, atol=2e-3)
-    o = ops.down_fp8(act, w_pj_q.to(device), pj_scale.to(device), ss.to(device), off.to(device), widen=False)
+    o = ops.down_fp8(act, w_pj_q.to(device), pj_scale.to(device), ss.to(device), off.to(device), widen=False, cfg=0)
     w_pj = oracle.dequant_fp8(w_pj_q, pj_scale)
     ref_o = oracle.scattered_experts_oracle(act.cpu(), w_pj, 1, se, ss, off, grouped_in=True)
     torch.testing.assert_close(o.cpu().float(), ref_o, rtol=2e-2, atol=2e-3)
@@ -433,8 +433,8 @@ def test_fp8_tiled_layout_is_bit_identical(device, T, E, k, H, I):
     ss, off = ss.to(device), off.to(device)
     fc_t = ops.fp8_tile(w_fc_q, glu=True)
     assert torch.equal(ops.fp8_untile(fc_t, E, 2 * I, H, True).view(torch.uint8), w_fc_q.view(torch.uint8))
-    act = ops.up_swiglu_fp8(x, w_fc_q, fc_scale, k, ss, off, widen=False)
-    act_t = ops.up_swiglu_fp8(x, fc_t, fc_scale, k, ss, off, widen=False)
+    act = ops.up_swiglu_fp8(x, w_fc_q, fc_scale, k, ss, off, widen=False, cfg=0)
+    act_t = ops.up_swiglu_fp8(x, fc_t, fc_scale, k, ss, off, widen=False, cfg=0)
     if H >= 512:
         assert torch.equal(act, act_t)
     else:  # row-major weights with a short K take the older kernel, which sums in another order
@@ -443,8 +443,8 @@ def test_fp8_tiled_layout_is_bit_identical(device, T, E, k, H, I):
     if I % 128 == 0:
         pj_t = ops.fp8_tile(w_pj_q, glu=False)
         assert torch.equal(ops.fp8_untile(pj_t, E, H, I, False).view(torch.uint8), w_pj_q.view(torch.uint8))
-        o = ops.down_fp8(act, w_pj_q, pj_scale, ss, off, widen=False)
-        o_t = ops.down_fp8(act, pj_t, pj_scale, ss, off, widen=False)
+        o = ops.down_fp8(act, w_pj_q, pj_scale, ss, off, widen=False, cfg=0)
+        o_t = ops.down_fp8(act, pj_t, pj_scale, ss, off, widen=False, cfg=0)
         if I >= 512:
             assert torch.equal(o, o_t)
         else:
@@ -475,15 +475,15 @@ def test_fp8_few_rows_per_expert(device, T, E, k, H, I, skew):
     print(f"fp8 few rows T={T} E={E} k={k} H={H} I={I} max rows {counts.max().item()}", flush=True)
     xd, ssd, offd = x.to(device), ss.to(device), off.to(device)
     fc_d, fcs_d, pj_d, pjs_d = (t.to(device) for t in (w_fc_q, fc_scale, w_pj_q, pj_scale))
-    act_t = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd, widen=False)
-    act_r = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False)
+    act_t = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd, widen=False, cfg=0)
+    act_r = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False, cfg=0)
     if H >= 512:
         assert torch.equal(act_t, act_r)
     ref_act = oracle.swiglu(oracle.scattered_experts_oracle(x, oracle.dequant_fp8(w_fc_q, fc_scale), k, se, ss, off,
                                                             grouped_out=True))
     torch.testing.assert_close(act_t.cpu().float(), ref_act, rtol=2e-2, atol=2e-3)
-    o_t = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd, widen=False)
-    o_r = ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd, widen=False)
+    o_t = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd, widen=False, cfg=0)
+    o_r = ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd, widen=False, cfg=0)
     if I >= 512:
         assert torch.equal(o_t, o_r)
     ref_o = oracle.scattered_experts_oracle(act_t.cpu(), oracle.dequant_fp8(w_pj_q, pj_scale), 1, se, ss, off,
@@ -544,10 +544,10 @@ def test_fp8_random_shapes(device, seed):
         xd, ssd, offd = x.to(device), ss.to(device), off.to(device)
         fc_d, fcs_d, pj_d, pjs_d = (t.to(device) for t in (w_fc_q, fc_scale, w_pj_q, pj_scale))
         print(f"fp8 random seed {seed} case {case}: T={T} E={E} k={k} H={H} I={I} {dtype}", flush=True)
-        act_t = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd, widen=False)
-        act_r = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False)
-        o_t = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd, widen=False)
-        o_r = ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd, widen=False)
+        act_t = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd, widen=False, cfg=0)
+        act_r = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False, cfg=0)
+        o_t = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd, widen=False, cfg=0)
+        o_r = ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd, widen=False, cfg=0)
         if H >= 512:
             assert torch.equal(act_t, act_r), (case, "up")
         if I >= 512:
@@ -601,10 +601,12 @@ def test_fp8_dequant_all_bit_patterns(device):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("T,E,k,H,I", [(300, 4, 2, 256, 128), (1024, 8, 2, 512, 272), (513, 3, 1, 384, 96)])
+@pytest.mark.parametrize("T,E,k,H,I", [(300, 4, 2, 256, 128), (1024, 8, 2, 512, 272), (513, 3, 1, 384, 96),
+                                       (1600, 2, 1, 256, 128)])
 def test_fp8_widened_weights_for_many_rows(device, dtype, T, E, k, H, I):
-    """From 80 rows per expert on the fp8 calls widen the weights and run the tiled 16-bit kernels: same contract
-    against the oracle, the automatic choice is the widened path, and it agrees with the fp8 kernels to rounding.
+    """With very many rows per expert the fp8 calls widen the weights and run the persistent 16-bit kernels: same
+    contract against the oracle, agreement with the fp8 kernels to rounding, and the automatic choice from 768 rows
+    per expert on.
     The widened weights are rounded to the activation dtype (2^-9 relative in bf16, beside the 2^-4 of e4m3 itself),
     which the fp8 kernels' weights are not: the absolute bound is twice that of the fp8 kernels' tests."""
     ops = _ops()
@@ -616,22 +618,65 @@ def test_fp8_widened_weights_for_many_rows(device, dtype, T, E, k, H, I):
     w_pj_q, pj_scale = oracle.quantize_fp8_per_channel(torch.randn(E, H, I, generator=g) * 0.02)
     xd, ssd, offd = x.to(device), ss.to(device), off.to(device)
     fc_d, fcs_d, pj_d, pjs_d = w_fc_q.to(device), fc_scale.to(device), w_pj_q.to(device), pj_scale.to(device)
-    assert T * k >= ops.FP8_DENSE_ROWS_PER_EXPERT * E
-    print(f"fp8 widened T={T} E={E} k={k} H={H} I={I} {dtype}", flush=True)
+    auto_widens = T * k >= ops.FP8_DENSE_ROWS_PER_EXPERT * E
+    print(f"fp8 widened T={T} E={E} k={k} H={H} I={I} {dtype} auto={auto_widens}", flush=True)
     act = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=True)
-    assert torch.equal(act, ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd))
+    auto = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd)
+    assert torch.equal(auto, act if auto_widens else ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False))
     ref_act = oracle.swiglu(oracle.scattered_experts_oracle(x, oracle.dequant_fp8(w_fc_q, fc_scale), k, se, ss, off,
                                                            grouped_out=True))
     torch.testing.assert_close(act.cpu().float(), ref_act, rtol=2e-2, atol=atol)
-    act_fp8 = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False)
+    act_fp8 = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False, cfg=0)
     torch.testing.assert_close(act.float(), act_fp8.float(), rtol=2e-2, atol=atol)
     o = ops.down_fp8(act, pj_d, pjs_d, ssd, offd, widen=True)
-    assert torch.equal(o, ops.down_fp8(act, pj_d, pjs_d, ssd, offd))
+    auto = ops.down_fp8(act, pj_d, pjs_d, ssd, offd)
+    assert torch.equal(auto, o if auto_widens else ops.down_fp8(act, pj_d, pjs_d, ssd, offd, widen=False))
     ref_o = oracle.scattered_experts_oracle(act.cpu(), oracle.dequant_fp8(w_pj_q, pj_scale), 1, se, ss, off,
                                             grouped_in=True)
     torch.testing.assert_close(o.cpu().float(), ref_o, rtol=2e-2, atol=atol)
-    o_fp8 = ops.down_fp8(act, pj_d, pjs_d, ssd, offd, widen=False)
+    o_fp8 = ops.down_fp8(act, pj_d, pjs_d, ssd, offd, widen=False, cfg=0)
     torch.testing.assert_close(o.float(), o_fp8.float(), rtol=2e-2, atol=atol)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k,H,I", [(8, 4, 1, 256, 128), (100, 4, 2, 1024, 208), (300, 4, 2, 256, 128),
+                                       (1024, 8, 2, 512, 272), (2100, 2, 1, 384, 112), (37, 16, 3, 2048, 640),
+                                       (600, 5, 1, 128, 80)])
+def test_fp8_tile_kernels(device, dtype, T, E, k, H, I):
+    """fp8 weights on the grouped GEMM's tile kernels (bytes widened on their way into LDS, scale in the epilogue):
+    the oracle's contract, bit-identical from the row-major and the tiled layout, equal to the streaming kernels up
+    to rounding; all three tile shapes (by rows per expert), partial K tiles, experts without rows.  The automatic
+    choice is the tile kernels from 16 rows per expert on average, the streaming kernels below."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(T * 3 + H + I)
+    se, ss, off = _routing(T, E, k, seed=T + 5)
+    x = _rand((T, H), 1.0, dtype, g)
+    w_fc_q, fc_scale = oracle.quantize_fp8_per_channel(torch.randn(E, 2 * I, H, generator=g) * 0.02)
+    w_pj_q, pj_scale = oracle.quantize_fp8_per_channel(torch.randn(E, H, I, generator=g) * 0.02)
+    xd, ssd, offd = x.to(device), ss.to(device), off.to(device)
+    fc_d, fcs_d, pj_d, pjs_d = w_fc_q.to(device), fc_scale.to(device), w_pj_q.to(device), pj_scale.to(device)
+    print(f"fp8 tiles T={T} E={E} k={k} H={H} I={I} {dtype}", flush=True)
+    act = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False, cfg=1)
+    ref_act = oracle.swiglu(oracle.scattered_experts_oracle(x, oracle.dequant_fp8(w_fc_q, fc_scale), k, se, ss, off,
+                                                           grouped_out=True))
+    torch.testing.assert_close(act.cpu().float(), ref_act, rtol=2e-2, atol=2e-3)
+    act_s = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False, cfg=0)
+    torch.testing.assert_close(act.float(), act_s.float(), rtol=2e-2, atol=2e-3)
+    if H % 128 == 0:
+        assert torch.equal(ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd, widen=False, cfg=1), act)
+    auto = ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False)
+    assert torch.equal(auto, act if T * k >= 16 * E else act_s)
+
+    o = ops.down_fp8(act, pj_d, pjs_d, ssd, offd, widen=False, cfg=1)
+    ref_o = oracle.scattered_experts_oracle(act.cpu(), oracle.dequant_fp8(w_pj_q, pj_scale), 1, se, ss, off,
+                                            grouped_in=True)
+    torch.testing.assert_close(o.cpu().float(), ref_o, rtol=2e-2, atol=2e-3)
+    o_s = ops.down_fp8(act, pj_d, pjs_d, ssd, offd, widen=False, cfg=0)
+    torch.testing.assert_close(o.float(), o_s.float(), rtol=2e-2, atol=2e-3)
+    if I % 128 == 0:
+        assert torch.equal(ops.down_fp8(act, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd, widen=False, cfg=1), o)
+    auto = ops.down_fp8(act, pj_d, pjs_d, ssd, offd, widen=False)
+    assert torch.equal(auto, o if T * k >= 16 * E else o_s)
 
 
 def test_inner_loop_probes_run(device):

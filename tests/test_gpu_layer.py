@@ -91,8 +91,8 @@ def test_layer_16bit(device, name, T):
 
 
 def test_layer_fp8_many_rows_per_expert(device):
-    """fp8 expert weights at a prefill-sized batch (192 rows per expert): the layer widens the weights for the call
-    and runs the tiled 16-bit kernels; same contract against the oracle as the decode batch."""
+    """fp8 expert weights at a prefill-sized batch (192 rows per expert): the fp8 calls run on the grouped GEMM's tile
+    kernels instead of the streaming kernels; same contract against the oracle as the decode batch."""
     import dataclasses
 
     w = dataclasses.replace(oracle.WORKLOADS["decode-fp8"], E=8, k=2, H=512, I=256, name="fp8-prefill")
