@@ -519,10 +519,14 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restri
 // 0.07 % of the products, so long groups beat groups of 3040 - 6080 rows (about four items per CU) by 4 - 7 %
 // under skewed loads and by 12 - 18 % under an even load (where no expert is split any more); the longest-first
 // plan keeps the few long items balanced.
-static int wgrad_chunk(int L, int M, int N) {
+static int wgrad_chunk(int L, int E, int M, int N) {
   const long tiles = (long)mi_ceil_div(M, 256) * mi_ceil_div(N, 256);
   long groups = (384 + tiles - 1) / tiles;
   long chunk = L / (groups > 0 ? groups : 1);
+  // With at least one item per CU from whole experts alone, an expert is only cut when it is half again as long as
+  // the average one: under an even load nobody is (no partial tiles, no second pass over them); the long experts of
+  // a skewed load still are.
+  if ((long)E * tiles >= 256 && chunk < 3L * (L / E) / 2) chunk = 3L * (L / E) / 2;
   if (chunk > 16384) chunk = 16384;
   if (chunk < 256) chunk = 256;
   return (int)(chunk / 32 * 32);
@@ -535,7 +539,7 @@ extern "C" size_t mi_moe_grouped_wgrad_workspace_bytes(int L, int E, int M, int 
   if (L < 1 || E < 1 || M < 1 || N < 1) return 0;
   // [partial slabs][plan: 32 ints (work counters, first slots) + one int per group + three per expert, padded to
   // 256 bytes]
-  const long groups = wgrad_max_groups(L, E, wgrad_chunk(L, M, N));
+  const long groups = wgrad_max_groups(L, E, wgrad_chunk(L, E, M, N));
   return (size_t)groups * (size_t)M * (size_t)N * sizeof(float) + wgrad_plan_bytes(groups, E);
 }
 
@@ -561,7 +565,7 @@ extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const v
   g.dw = dw;
   g.next_item = nullptr;
   g.L = L; g.M = M; g.N = N; g.E = E;
-  g.chunk = wgrad_chunk(L, M, N);
+  g.chunk = wgrad_chunk(L, E, M, N);
   const long max_groups = wgrad_max_groups(L, E, g.chunk);
   const int red_at = (int)(32 + max_groups);
   if (L > 0) {
