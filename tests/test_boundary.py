@@ -81,6 +81,11 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_router_dlogits(None, None, None, None, 0, 8, 2, _lib.F32, None, None) == 0
     assert lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) > 0
     assert lib.mi_moe_router_fused_workspace_bytes(32768, 1536, 40) == 0
+    # the few-token forms end at 384 tokens where the gate weights fit in LDS, at 1024 where they do not
+    assert lib.mi_moe_router_fused_workspace_bytes(384, 1536, 40) > 0
+    assert lib.mi_moe_router_fused_workspace_bytes(385, 1536, 40) == 0
+    assert lib.mi_moe_router_fused_workspace_bytes(1024, 4096, 64) > 0
+    assert lib.mi_moe_router_fused_workspace_bytes(1025, 4096, 64) == 0
     assert lib.mi_moe_router_fused_sort_workspace_bytes(64, 4096, 64, 6) == lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) + 256
     assert lib.mi_moe_router_fused_sort_workspace_bytes(2048, 4096, 64, 8) == 0   # many tokens, gate weights beyond LDS
     assert lib.mi_moe_router_fused_sort_workspace_bytes(1024, 1024, 64, 9) == 0   # T * k beyond the one-block sort
@@ -137,6 +142,16 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_fp8_tiled_bytes(64, 4096, 1408, 0) == 64 * 4096 * 1408
     assert lib.mi_moe_fp8_tiled_bytes(4, 20, 256, 1) == 4 * 2 * 2 * 4096  # 20 channels pad to two units
     assert lib.mi_moe_fp8_tiled_bytes(4, 20, 200, 1) == 0
+    # the same calls with the kernel family chosen by the caller, and the widening pass
+    assert lib.mi_moe_up_swiglu_fp8_cfg(None, None, None, None, None, None, 16, 64, 32, 4, 2, _lib.BF16, 0, 2, None) == E_UNSUP
+    assert lib.mi_moe_up_swiglu_fp8_cfg(None, None, None, None, None, None, 16, 64, 32, 4, 2, _lib.BF16, 0, 1, None) == E_NULL
+    assert lib.mi_moe_down_fp8_cfg(None, None, None, None, None, None, 16, 64, 32, 4, _lib.BF16, 0, -2, None) == E_UNSUP
+    assert lib.mi_moe_down_fp8_cfg(None, None, None, None, None, None, 0, 64, 32, 4, _lib.BF16, 0, 1, None) == 0
+    assert lib.mi_moe_fp8_dequant(None, None, None, 4, 32, 64, 1, 0, _lib.F32, None) == E_DTYPE
+    assert lib.mi_moe_fp8_dequant(None, None, None, 4, 32, 72, 1, 0, _lib.BF16, None) == E_UNSUP   # in % 16
+    assert lib.mi_moe_fp8_dequant(None, None, None, 4, 32, 64, 1, 1, _lib.BF16, None) == E_UNSUP   # tiled: in % 128
+    assert lib.mi_moe_fp8_dequant(None, None, None, 4, 32, 128, 1, 1, _lib.BF16, None) == E_NULL
+    assert lib.mi_moe_fp8_dequant(None, None, None, 0, 32, 128, 1, 1, _lib.BF16, None) == E_SHAPE
     # backward entry points
     assert lib.mi_moe_scattered_gemm_wt(None, None, None, None, None, 16, 128, 8, 4, 2, 0, 1, _lib.F32, None) == E_NULL
     assert lib.mi_moe_scattered_gemm_wt(None, None, None, None, None, 0, 128, 8, 4, 2, 0, 1, _lib.BF16, None) == 0
