@@ -523,7 +523,8 @@ def test_fp8_random_shapes(device, seed):
     """The fp8 kernels on random shapes and routings: 1 to 257 tokens, 1 to 64 experts (some without rows, some with
     many times 8), hidden and intermediate sizes from 128 to 2048 in steps of 128 (one to sixteen ring stages, so
     both the short-ring path and the counted tail), both 16-bit types.  Tiled and row-major weights must agree bit
-    for bit where both run the streaming kernel (K >= 512), and both must match the oracle."""
+    for bit where both run the streaming kernel (K >= 512), and both must match the oracle; the tile kernels run
+    the same problems (bit-identical from either weight layout, same bounds against the oracle)."""
     import random
 
     ops = _ops()
@@ -556,8 +557,14 @@ def test_fp8_random_shapes(device, seed):
                                                                 grouped_out=True))
         ref_o = oracle.scattered_experts_oracle(act_t.cpu(), oracle.dequant_fp8(w_pj_q, pj_scale), 1, se, ss, off,
                                                 grouped_in=True)
+        # the tile kernels on the same problem (tiled and row-major weights: the same bits)
+        act_k = ops.up_swiglu_fp8(xd, ops.fp8_tile(fc_d, glu=True), fcs_d, k, ssd, offd, widen=False, cfg=1)
+        assert torch.equal(act_k, ops.up_swiglu_fp8(xd, fc_d, fcs_d, k, ssd, offd, widen=False, cfg=1)), (case, "up tiles")
+        o_k = ops.down_fp8(act_t, ops.fp8_tile(pj_d, glu=False), pjs_d, ssd, offd, widen=False, cfg=1)
+        assert torch.equal(o_k, ops.down_fp8(act_t, pj_d, pjs_d, ssd, offd, widen=False, cfg=1)), (case, "down tiles")
         for name, got, ref in (("up", act_t, ref_act), ("up row-major", act_r, ref_act), ("down", o_t, ref_o),
-                               ("down row-major", o_r, ref_o)):
+                               ("down row-major", o_r, ref_o), ("up tile kernels", act_k, ref_act),
+                               ("down tile kernels", o_k, ref_o)):
             err = (got.cpu().float() - ref).abs().max().item()
             assert err <= 2e-2 * ref.abs().max().item() + 2e-3, (case, name, err)
 
