@@ -155,11 +155,18 @@ struct RouterNorm {
 // in one turn are consecutive -- a chunk of nwaves * 16 tokens -- so the workgroup counts the experts its
 // waves select in LDS and writes chunk_hist[e * nchunks + chunk], the layout the sort's scan pass reads; the sort
 // then needs neither its histogram launch nor that launch's read of the expert ids.
-template <typename T, int DEPTH, bool NORM>
+// KS (few groups per workgroup: every group is walked in one turn): `ksplit` waves share a group and split its K
+// steps (wave part p takes steps p, p + ksplit, ...), so that a group's row is walked in one or two round trips to
+// memory instead of four; the partial logits meet in LDS (over the weights, which nobody needs any more, or behind
+// them when they are smaller than the 32 KB this takes: `red_at`) and are added in part order.  Measured, hidden
+// 1536, 40 experts: 13.0 us for this kernel from 1024 to 4096 tokens (20.5 - 20.9 us with one wave per group),
+// 16.3 us at 8192, 21.8 us at 16384 tokens.
+template <typename T, int DEPTH, bool NORM, bool KS = false>
 __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ gw, const float* __restrict__ bias, int Trows, int H, int E, int k,
     T* __restrict__ logits_out, T* __restrict__ gates, int32_t* __restrict__ idx, RouterNorm norm,
-    int32_t* __restrict__ chunk_hist, int nchunks, int nwaves) {
+    int32_t* __restrict__ chunk_hist, int nchunks, int nwaves, int ksplit, int red_at) {
+  static_assert(!(KS && NORM), "the K split is built for the form without the norm");
   typedef typename RMfma<T>::vec frag_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char wlds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -169,16 +176,21 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
   const int nsteps = (H + 63) >> 6;
   const int ngroups = (Trows + 15) >> 4;
   const int stride = gridDim.x * nwaves;
-  int grp = wave < nwaves ? blockIdx.x * nwaves + wave : ngroups;
+  // KS: wave = slot * ksplit + part
+  const int part = KS ? wave % ksplit : 0;
+  const int slot = KS ? wave / ksplit : wave;
+  const int kstep = KS ? ksplit : 1;
+  const int nmine = KS ? (nsteps - part + ksplit - 1) / ksplit : nsteps;  // K steps of this wave
+  int grp = slot < nwaves ? blockIdx.x * nwaves + slot : ngroups;
 
   // x ring of the wave's current group; the first DEPTH steps of a group are requested before the previous
   // group's epilogue (for the first group: before the weights are copied), so their latency is hidden
   const T* xrow = x;
   u32x4 xr[DEPTH][2];
-  auto load_x = [&](int step, u32x4 (&dst)[2]) {
-    const int kpos = step * 64 + q * 16;
+  auto load_x = [&](int step, u32x4 (&dst)[2]) {  // step: the wave's own count; K step step * kstep + part
+    const int kpos = (step * kstep + part) * 64 + q * 16;
     dst[0] = dst[1] = (u32x4){0u, 0u, 0u, 0u};
-    if (step < nsteps && kpos < H) {  // the MFMA runs on all lanes: out-of-range k contributes zeros
+    if (step < nmine && kpos < H) {  // the MFMA runs on all lanes: out-of-range k contributes zeros
       // Ordinary (cached) loads: with the norm the rows are read twice, and without it they are read again right
       // after, as the gathered operand of the up-projection -- which runs 1 - 1.5 % faster on rows this pass left in
       // the caches than on rows streamed through with the non-temporal policy (and this kernel is no slower).
@@ -236,9 +248,13 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
     wbase[eb] = e * pitch;
   }
   // with a histogram every wave walks the same number of turns (a turn ends in workgroup barriers)
-  const int nturns = chunk_hist != nullptr ? (ngroups + stride - 1) / stride : 0;
-  for (int turn = 0; chunk_hist != nullptr ? turn < nturns : grp < ngroups; ++turn) {
-    if (grp < ngroups) {
+  const int nturns = KS ? 1 : (chunk_hist != nullptr ? (ngroups + stride - 1) / stride : 0);
+  for (int turn = 0; (KS || chunk_hist != nullptr) ? turn < nturns : grp < ngroups; ++turn) {
+    const bool active = grp < ngroups;
+    f32x4 acc[4];
+#pragma unroll
+    for (int eb = 0; eb < 4; ++eb) acc[eb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    if (active) {
     float rstd = 1.0f;
     if (NORM) {
       // first pass over the group's rows: sum of squares of the 16 k this lane holds per step, then over the
@@ -271,20 +287,18 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
       const int t = grp * 16 + r;
       if (t < Trows) xn_row = static_cast<T*>(norm.xnorm_out) + (size_t)t * H;
     }
-    f32x4 acc[4];
-#pragma unroll
-    for (int eb = 0; eb < 4; ++eb) acc[eb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < nsteps; s0 += DEPTH) {
+    for (int s0 = 0; s0 < nmine; s0 += DEPTH) {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
         const int step = s0 + d;
-        if (step < nsteps) {
-          const int kbyte = (step * 64 + q * 16) * (int)sizeof(T);
-          const bool valid = step * 64 + q * 16 < H;
+        if (step < nmine) {
+          const int kel = (step * kstep + part) * 64 + q * 16;
+          const int kbyte = kel * (int)sizeof(T);
+          const bool valid = kel < H;
           u32x4 x0 = xr[d][0], x1 = xr[d][1];
           load_x(step + DEPTH, xr[d]);
           if (NORM && valid) {
-            const int kpos = step * 64 + q * 16;
+            const int kpos = kel;
             const f32x4* g4 = reinterpret_cast<const f32x4*>(glds + kpos);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -313,11 +327,35 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
         }
       }
     }
-    const int t = grp * 16 + r;
-    grp += stride;
-    if (grp < ngroups) open_group(grp);
-    router_epilogue<T>(acc, t, t < Trows, q, bias, E, k, logits_out, gates, idx,
-                       chunk_hist != nullptr ? whist : nullptr);
+    }
+    if constexpr (KS) {
+      // every wave is done with the weights; the parts of a group meet in LDS and part 0 adds them in part order
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      f32x4* red = reinterpret_cast<f32x4*>(wlds + red_at);
+      if (part != 0) {
+#pragma unroll
+        for (int eb = 0; eb < 4; ++eb) red[(wave * 4 + eb) * 64 + lane] = acc[eb];
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (part == 0) {
+        for (int p = 1; p < ksplit; ++p) {
+#pragma unroll
+          for (int eb = 0; eb < 4; ++eb) acc[eb] += red[((wave + p) * 4 + eb) * 64 + lane];
+        }
+      }
+    }
+    if (active && part == 0) {
+      const int t = grp * 16 + r;
+      grp += stride;
+      if (!KS && grp < ngroups) open_group(grp);
+      router_epilogue<T>(acc, t, t < Trows, q, bias, E, k, logits_out, gates, idx,
+                         chunk_hist != nullptr ? whist : nullptr);
     } else {
       grp += stride;
     }
@@ -711,13 +749,31 @@ static int launch_router_lds(const void* x, const void* gw, const float* bias, i
   int blocks = 0, waves = 0;
   int rc = router_lds_shape(T_, &blocks, &waves);
   if (rc != MI_MOE_OK) return rc;
-  auto kern = waves > 4 ? router_fused_lds_kernel<T, 3, NORM> : router_fused_lds_kernel<T, 6, NORM>;
+  // few groups per workgroup (at most four waves would walk one): the idle waves take shares of the K steps
+  // (router_fused_lds_kernel, KS); 3 groups leave two waves without a share
+  constexpr bool CAN_SPLIT = !NORM;
+  const int ksplit = (CAN_SPLIT && waves <= 4) ? (waves == 1 ? 8 : (waves == 2 ? 4 : 2)) : 1;
+  size_t bytes = lds + (size_t)E * sizeof(int);
+  int red_at = 0;
+  if (ksplit > 1) {
+    constexpr size_t RED_BYTES = (size_t)ROUTER_LDS_WAVES * 4 * 64 * sizeof(f32x4);  // 32 KB
+    if ((size_t)E * ((size_t)H * sizeof(T) + 16) < RED_BYTES) {  // small weights: behind everything else
+      red_at = (int)((bytes + 15) / 16 * 16);
+      bytes = (size_t)red_at + RED_BYTES;
+    }
+  }
+  void (*kern)(const T*, const T*, const float*, int, int, int, int, T*, T*, int32_t*, RouterNorm, int32_t*, int, int, int,
+               int);
+  int slot;
+  if (waves > 4) { kern = router_fused_lds_kernel<T, 3, NORM, false>; slot = 0; }
+  else if constexpr (CAN_SPLIT) { kern = router_fused_lds_kernel<T, 6, false, true>; slot = 1; }
+  else { kern = router_fused_lds_kernel<T, 6, NORM, false>; slot = 1; }
   static std::atomic<uint64_t> lds_ok[2];  // the LDS size varies with E and H: opt in to the most it can be
-  rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok[waves > 4 ? 1 : 0]);
+  rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok[slot]);
   if (rc != MI_MOE_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(ROUTER_LDS_WAVES * 64), lds + (size_t)E * sizeof(int), s,
-                     static_cast<const T*>(x), static_cast<const T*>(gw), bias, T_, H, E, k,
-                     static_cast<T*>(logits_out), static_cast<T*>(gates), idx, norm, chunk_hist, nchunks, waves);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(ROUTER_LDS_WAVES * 64), bytes, s, static_cast<const T*>(x),
+                     static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out), static_cast<T*>(gates), idx,
+                     norm, chunk_hist, nchunks, waves, ksplit, red_at);
   return mi_launch_status();
 }
 
