@@ -703,9 +703,9 @@ static bool router_lds_fits(int H, int E) { return (size_t)E * ((size_t)H * 2 + 
 // The few-token forms (K split across waves or workgroups) are used up to ROUTER_FEW_TOKENS tokens, and up to 1024
 // where the LDS-resident kernel does not take the gate weights.  Every entry point applies the same rule, so that
 // the router gives the same bits whichever of them a caller uses.  Measured, router + sort as the layer calls them,
-// hidden size 1536, 40 experts, top-8: few-token form 22.5 / 26 / 35 / 43 us at 384 / 512 / 768 / 1024 tokens (its
-// one-block sort is what grows), LDS-resident kernel + scan + scatter 24.6 us from 192 to 2048 tokens.
-#define ROUTER_FEW_TOKENS 384
+// hidden size 1536, 40 experts, top-8: few-token form 19.2 / 22.5 / 26 / 35 / 43 us at 256 / 384 / 512 / 768 / 1024
+// tokens (its one-block sort is what grows), LDS-resident kernel + scan + scatter 21.4 us from 320 to 4096 tokens.
+#define ROUTER_FEW_TOKENS 320
 static bool router_few_tokens(int T_, int H, int E) { return T_ <= (router_lds_fits(H, E) ? ROUTER_FEW_TOKENS : 1024); }
 
 static size_t router_ws_bytes(int T_, int H, int E) {

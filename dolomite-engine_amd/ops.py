@@ -192,7 +192,7 @@ def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch
 
 def router_fused_sort_supported(x: torch.Tensor, num_experts: int, k: int) -> bool:
     """Whether :func:`router_fused_sort` takes the shape: few tokens (split-K router whose finishing launch sorts,
-    T <= 384, or T <= 1024 with T * k <= 8192 where the gate weights do not fit in LDS), or gate weights that fit
+    T <= 320, or T <= 1024 with T * k <= 8192 where the gate weights do not fit in LDS), or gate weights that fit
     in LDS (the router counts the experts for the sort's two remaining passes)."""
     if not (_router_streaming_supported(x, num_experts, k) and x.is_cuda and x.dim() == 2 and x.shape[0] >= 1):
         return False

@@ -81,9 +81,9 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_router_dlogits(None, None, None, None, 0, 8, 2, _lib.F32, None, None) == 0
     assert lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) > 0
     assert lib.mi_moe_router_fused_workspace_bytes(32768, 1536, 40) == 0
-    # the few-token forms end at 384 tokens where the gate weights fit in LDS, at 1024 where they do not
-    assert lib.mi_moe_router_fused_workspace_bytes(384, 1536, 40) > 0
-    assert lib.mi_moe_router_fused_workspace_bytes(385, 1536, 40) == 0
+    # the few-token forms end at 320 tokens where the gate weights fit in LDS, at 1024 where they do not
+    assert lib.mi_moe_router_fused_workspace_bytes(320, 1536, 40) > 0
+    assert lib.mi_moe_router_fused_workspace_bytes(321, 1536, 40) == 0
     assert lib.mi_moe_router_fused_workspace_bytes(1024, 4096, 64) > 0
     assert lib.mi_moe_router_fused_workspace_bytes(1025, 4096, 64) == 0
     assert lib.mi_moe_router_fused_sort_workspace_bytes(64, 4096, 64, 6) == lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) + 256
