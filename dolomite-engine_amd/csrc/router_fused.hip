@@ -155,18 +155,18 @@ struct RouterNorm {
 // in one turn are consecutive -- a chunk of nwaves * 16 tokens -- so the workgroup counts the experts its
 // waves select in LDS and writes chunk_hist[e * nchunks + chunk], the layout the sort's scan pass reads; the sort
 // then needs neither its histogram launch nor that launch's read of the expert ids.
-// KS (few groups per workgroup: every group is walked in one turn): `ksplit` waves share a group and split its K
+// KS (at most four groups per workgroup: every group is walked in one turn): `ksplit` waves share a group and split its K
 // steps (wave part p takes steps p, p + ksplit, ...), so that a group's row is walked in one or two round trips to
 // memory instead of four; the partial logits meet in LDS (over the weights, which nobody needs any more, or behind
 // them when they are smaller than the 32 KB this takes: `red_at`) and are added in part order.  Measured, hidden
 // 1536, 40 experts: 13.0 us for this kernel from 1024 to 4096 tokens (20.5 - 20.9 us with one wave per group),
-// 16.3 us at 8192, 21.8 us at 16384 tokens.
+// 16.3 us at 8192, 21.8 us at 16384 tokens.  With the norm folded in, the sums of squares of a row's parts meet in
+// LDS first (`ss_at`): 31.5 / 32.8 / 46.7 -> 15.2 / 17.2 / 35.5 us at 1024 / 4096 / 16384 tokens.
 template <typename T, int DEPTH, bool NORM, bool KS = false>
 __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ gw, const float* __restrict__ bias, int Trows, int H, int E, int k,
     T* __restrict__ logits_out, T* __restrict__ gates, int32_t* __restrict__ idx, RouterNorm norm,
-    int32_t* __restrict__ chunk_hist, int nchunks, int nwaves, int ksplit, int red_at) {
-  static_assert(!(KS && NORM), "the K split is built for the form without the norm");
+    int32_t* __restrict__ chunk_hist, int nchunks, int nwaves, int ksplit, int red_at, int ss_at) {
   typedef typename RMfma<T>::vec frag_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char wlds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -254,17 +254,15 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
     f32x4 acc[4];
 #pragma unroll
     for (int eb = 0; eb < 4; ++eb) acc[eb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    if (active) {
-    float rstd = 1.0f;
-    if (NORM) {
-      // first pass over the group's rows: sum of squares of the 16 k this lane holds per step, then over the
-      // four lanes of the token
-      float ss = 0.f;
-      for (int s0 = 0; s0 < nsteps; s0 += DEPTH) {
+    float ss = 0.f, rstd = 1.0f;
+    if (NORM && active) {
+      // first pass over the group's rows (KS: over this wave's K steps of them): sum of squares of the 16 k this
+      // lane holds per step, then over the four lanes of the token
+      for (int s0 = 0; s0 < nmine; s0 += DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
           const int step = s0 + d;
-          if (step < nsteps) {
+          if (step < nmine) {
             const u32x4 x0 = xr[d][0], x1 = xr[d][1];
             load_x(step + DEPTH, xr[d]);
 #pragma unroll
@@ -278,10 +276,22 @@ __global__ __launch_bounds__(ROUTER_LDS_WAVES * 64) void router_fused_lds_kernel
       }
       ss += __shfl_xor(ss, 16, MI_WAVE);
       ss += __shfl_xor(ss, 32, MI_WAVE);
-      rstd = 1.0f / sqrtf(ss / (float)H + norm.eps);
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) load_x(d, xr[d]);  // second pass, out of L2
     }
+    if constexpr (NORM && KS) {
+      // the parts of a row's sum of squares meet in LDS and every wave of the group adds them in part order
+      float* ssred = reinterpret_cast<float*>(wlds + ss_at);
+      if (q == 0) ssred[wave * 16 + r] = ss;
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the x loads of the second pass stay in flight
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      ss = 0.f;
+      for (int p = 0; p < ksplit; ++p) ss += ssred[(wave - part + p) * 16 + r];
+    }
+    if (NORM) rstd = 1.0f / sqrtf(ss / (float)H + norm.eps);
+    if (active) {
     T* xn_row = nullptr;
     if (NORM) {
       const int t = grp * 16 + r;
@@ -751,10 +761,13 @@ static int launch_router_lds(const void* x, const void* gw, const float* bias, i
   if (rc != MI_MOE_OK) return rc;
   // few groups per workgroup (at most four waves would walk one): the idle waves take shares of the K steps
   // (router_fused_lds_kernel, KS); 3 groups leave two waves without a share
-  constexpr bool CAN_SPLIT = !NORM;
-  const int ksplit = (CAN_SPLIT && waves <= 4) ? (waves == 1 ? 8 : (waves == 2 ? 4 : 2)) : 1;
+  const int ksplit = waves <= 4 ? (waves == 1 ? 8 : (waves == 2 ? 4 : 2)) : 1;
   size_t bytes = lds + (size_t)E * sizeof(int);
-  int red_at = 0;
+  int red_at = 0, ss_at = 0;
+  if (NORM && ksplit > 1) {  // 16 partial sums of squares per wave
+    ss_at = (int)((bytes + 15) / 16 * 16);
+    bytes = (size_t)ss_at + ROUTER_LDS_WAVES * 16 * sizeof(float);
+  }
   if (ksplit > 1) {
     constexpr size_t RED_BYTES = (size_t)ROUTER_LDS_WAVES * 4 * 64 * sizeof(f32x4);  // 32 KB
     if ((size_t)E * ((size_t)H * sizeof(T) + 16) < RED_BYTES) {  // small weights: behind everything else
@@ -762,18 +775,14 @@ static int launch_router_lds(const void* x, const void* gw, const float* bias, i
       bytes = (size_t)red_at + RED_BYTES;
     }
   }
-  void (*kern)(const T*, const T*, const float*, int, int, int, int, T*, T*, int32_t*, RouterNorm, int32_t*, int, int, int,
-               int);
-  int slot;
-  if (waves > 4) { kern = router_fused_lds_kernel<T, 3, NORM, false>; slot = 0; }
-  else if constexpr (CAN_SPLIT) { kern = router_fused_lds_kernel<T, 6, false, true>; slot = 1; }
-  else { kern = router_fused_lds_kernel<T, 6, NORM, false>; slot = 1; }
+  auto kern = waves > 4 ? router_fused_lds_kernel<T, 3, NORM, false> : router_fused_lds_kernel<T, 6, NORM, true>;
+  const int slot = waves > 4 ? 0 : 1;
   static std::atomic<uint64_t> lds_ok[2];  // the LDS size varies with E and H: opt in to the most it can be
   rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), MI_LDS_MAX_BYTES, lds_ok[slot]);
   if (rc != MI_MOE_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(ROUTER_LDS_WAVES * 64), bytes, s, static_cast<const T*>(x),
                      static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out), static_cast<T*>(gates), idx,
-                     norm, chunk_hist, nchunks, waves, ksplit, red_at);
+                     norm, chunk_hist, nchunks, waves, ksplit, red_at, ss_at);
   return mi_launch_status();
 }
 
