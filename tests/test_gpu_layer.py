@@ -486,3 +486,66 @@ def test_training_and_inference_route_tied_rows_alike(device, dtype):
     assert torch.equal(idx_eval.cpu().long(), want), "inference-mode routing is not the canonical one"
     ulp = {torch.bfloat16: 8e-3, torch.float32: 2e-6}[dtype]  # torch's softmax and the kernel's differ by a rounding
     torch.testing.assert_close(gates.detach().float(), gates_eval.float(), rtol=ulp, atol=ulp * 0.1)
+
+
+@pytest.mark.parametrize("seed", list(range(16)))
+def test_training_random_shapes(device, seed):
+    """Training through the kernel branch at random shapes (token counts around the kernels' tile and dispatch
+    boundaries, hidden and intermediate sizes that are multiples of 8 only, 2 to 72 experts, with and without
+    shared experts, the pre-activation kept or recomputed): output, aux loss and every gradient against torch
+    autograd through the eager branch of the same module, each relative to its largest entry.  k >= 2 and no fp16:
+    with one expert per token only the aux loss reaches the gate weights, and the eager branch's 16-bit aux loss
+    is the less exact side of that comparison."""
+    import random
+
+    from dolomite_engine_amd import Kernel, MoE, enable_kernels
+    from dolomite_engine_amd.loss import clear_aux_loss, get_aux_loss
+
+    rng = random.Random(1000 + seed)
+    dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float32])
+    T = rng.choice([2, 15, 17, 63, 65, 300, 321, 1000, 1025, 2500, 4100]) if rng.random() < 0.5 else rng.randint(2, 3000)
+    H = 8 * rng.randint(2, 160) if rng.random() < 0.7 else 32 * rng.randint(1, 48)
+    E = rng.choice([2, 3, 7, 8, 16, 17, 32, 40, 64, 65, 72])
+    k = rng.randint(2, min(E, 8))
+    I = 8 * rng.randint(1, 96) if rng.random() < 0.7 else 64 * rng.randint(1, 12)
+    shared = rng.choice([None, None, 8 * rng.randint(1, 40)])
+    activation = rng.choice(["swiglu", "swiglu", "swiglu", "gelu_pytorch_tanh", "geglu"])
+    keep = rng.random() < 0.6
+    print(f"training {dtype} T={T} H={H} E={E} k={k} I={I} shared={shared} {activation} keep={keep}", flush=True)
+    torch.manual_seed(seed)
+    m = MoE(hidden_size=H, intermediate_size=I, shared_intermediate_size=shared, num_experts=E,
+            num_experts_per_tok=k, activation_function=activation, add_bias=False, dropout=0.0, init_method="normal",
+            initializer_range=0.1, m_width=None, num_layers=1, use_padding_free_transformer=True)
+    m = m.to(dtype).to(device).train()
+    m.keep_preactivation = keep
+    x0 = torch.randn(T, H, device=device, dtype=dtype)
+    dy = torch.randn(T, H, device=device, dtype=dtype)
+    with torch.no_grad():
+        idx_e = m._compute_routing_weights(x0)[2].long().sort(dim=1).values
+        with enable_kernels([Kernel.scattermoe]):
+            idx_k = m._compute_routing_weights(x0)[2].long().sort(dim=1).values
+    if not torch.equal(idx_e, idx_k):  # a logit on a rounding boundary of the model dtype: the branches route apart
+        pytest.skip("the two branches' logits round a selection boundary differently on this seed")
+
+    def run(kernels):
+        m.zero_grad(set_to_none=True)
+        clear_aux_loss()
+        x = x0.clone().requires_grad_(True)
+        if kernels:
+            with enable_kernels([Kernel.scattermoe]):
+                y = m(x)
+        else:
+            y = m(x)
+        aux = get_aux_loss()
+        ((y * dy).sum() + 0.01 * aux).backward()
+        return y.detach(), aux.detach(), x.grad.detach(), {n: p.grad.detach().clone() for n, p in m.named_parameters()}
+
+    y_e, aux_e, dx_e, g_e = run(False)
+    y_k, aux_k, dx_k, g_k = run(True)
+    tol = {torch.float32: 2e-3, torch.bfloat16: 5e-2}[dtype]
+    torch.testing.assert_close(aux_k.float(), aux_e.float(), rtol=1e-4 if dtype == torch.float32 else 2e-2, atol=1e-5)
+    assert set(g_k) == set(g_e)
+    for name, got, want in [("y", y_k, y_e), ("dx", dx_k, dx_e)] + [(n, g_k[n], g_e[n]) for n in g_e]:
+        scale = want.float().abs().max().clamp_min(1e-6)
+        err = ((got.float() - want.float()).abs().max() / scale).item()
+        assert err <= tol, f"{name}: {err:.3e} of the largest entry"
