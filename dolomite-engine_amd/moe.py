@@ -382,10 +382,22 @@ class MoE(nn.Module):
             elif self.c_fc.weight_q is not None:
                 if not self._fused_swiglu:
                     raise RuntimeError("fp8 expert weights need the swiglu activation")
-                hidden_states = ops.up_swiglu_fp8(hidden_states, self.c_fc.weight_q, self.c_fc.weight_scale,
-                                                  self.top_k, sorted_scattered_idxs, expert_offsets)
-                hidden_states = ops.down_fp8(hidden_states, self.c_proj.weight_q, self.c_proj.weight_scale,
-                                             sorted_scattered_idxs, expert_offsets)
+                if self.hidden_size % 16 or self.intermediate_size % 16:
+                    # the fp8 kernels read the weights 16 at a time: other sizes run the 16-bit kernels on weights
+                    # widened for the call (round(w * scale), what the eager branch multiplies with)
+                    ops._warn_once(("fp8_widened", self.hidden_size, self.intermediate_size),
+                                   f"MoE with fp8 expert weights, hidden size {self.hidden_size}, intermediate size "
+                                   f"{self.intermediate_size}: the fp8 kernels need multiples of 16; widening the "
+                                   "weights on every call")
+                    hidden_states = ops.up_swiglu(hidden_states, self.c_fc.dense_weight(), self.top_k,
+                                                  sorted_scattered_idxs, expert_offsets)
+                    hidden_states = ops.scattered_gemm(hidden_states, self.c_proj.dense_weight(), 1,
+                                                       sorted_scattered_idxs, expert_offsets, True, False)
+                else:
+                    hidden_states = ops.up_swiglu_fp8(hidden_states, self.c_fc.weight_q, self.c_fc.weight_scale,
+                                                      self.top_k, sorted_scattered_idxs, expert_offsets)
+                    hidden_states = ops.down_fp8(hidden_states, self.c_proj.weight_q, self.c_proj.weight_scale,
+                                                 sorted_scattered_idxs, expert_offsets)
                 hidden_states = ops.combine(hidden_states, router_weights, shared, residual, residual_scale)
             else:
                 if self._fused_swiglu:

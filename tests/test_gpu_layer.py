@@ -99,6 +99,18 @@ def test_layer_fp8_many_rows_per_expert(device):
     _check_layer(w, 768, device, dict(rtol=2e-2, atol=2e-2))
 
 
+@pytest.mark.parametrize("H,I", [(264, 256), (256, 152), (72, 40)])
+def test_layer_fp8_sizes_not_multiples_of_16(device, H, I):
+    """fp8 expert weights with a hidden or intermediate size that the fp8 kernels do not read (they take the
+    weights 16 at a time): the module widens the weights for the call and runs the 16-bit kernels; same contract
+    against the oracle."""
+    import dataclasses
+
+    w = dataclasses.replace(oracle.WORKLOADS["decode-fp8"], E=8, k=2, H=H, I=I, name="fp8-odd-sizes")
+    with pytest.warns(RuntimeWarning, match="multiples of 16"):
+        _check_layer(w, 300, device, dict(rtol=2e-2, atol=2e-2))
+
+
 def test_layer_mixtral_shape_reduced_experts(device):
     """Mixtral-shape contraction sizes (H=4096, I=14336) with 2 experts so the CPU oracle stays small."""
     import dataclasses
