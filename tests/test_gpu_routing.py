@@ -353,6 +353,11 @@ def test_routing_random_shapes(device, seed):
         ref_logits = oracle.router_logits(x, w, b)
         tol = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.bfloat16: dict(rtol=1.6e-2, atol=2e-3),
                torch.float16: dict(rtol=2e-3, atol=1e-3)}[dtype]
+        if b is not None and dtype != torch.float32:
+            # the product is rounded before the bias is added: where the two cancel, one rounding step of the
+            # product is large against the sum
+            step = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+            tol["atol"] += step * float((ref_logits.float() - b).abs().max())
         torch.testing.assert_close(logits.cpu().float(), ref_logits.float(), **tol)
         vals, ref_idx = oracle.topk_canonical(logits.cpu(), k)
         assert torch.equal(idx.cpu().long(), ref_idx), case
