@@ -894,8 +894,25 @@ extern "C" int mi_moe_router_fused_sort(const void* x, const void* gate_w, const
   return mi_sort_after_hist(idx_out, T * k, E, chunk_tokens * k, sorted_expert, sorted_scattered, expert_offsets, hist, s);
 }
 
+// Many tokens and more than 64 experts (16-bit, no bias): the logits are a product of a size that wants the
+// grouped GEMM's tile kernels -- the general kernel re-reads all gate weights from L2 for every 16 tokens.  With
+// a workspace the router runs that kernel with ONE expert that owns every row (x rows in place, gate_w as its
+// (1, E, H) weight: fp32 accumulation, one rounding, as F.linear), then the top-k kernel on the logits -- in
+// logits_out when the caller wants them, else in the workspace.  Measured, 32768 tokens: 128 experts, hidden
+// 2048, 177 -> 47 us; 256 experts, hidden 7168, 951 -> 194 us; the crossover is near T * E = 2^20.
+static bool router_gemm_form(int T_, int H, int E, int k, int dtype, const float* bias) {
+  return dtype != MI_MOE_F32 && bias == nullptr && E > 64 && (long)T_ * E >= (1L << 20) && H % 16 == 0;
+}
+static size_t router_gemm_form_bytes(int T_, int E) { return ((size_t)T_ * E * 2 + 255) / 256 * 256 + 256; }
+
+__global__ void router_one_expert_offsets_kernel(int32_t* offsets, int rows) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) offsets[0] = rows;
+}
+
 extern "C" size_t mi_moe_router_fused_workspace_bytes(int T, int H, int E) {
-  return (T < 0 || H < 1 || E < 1) ? 0 : router_ws_bytes(T, H, E);
+  if (T < 0 || H < 1 || E < 1) return 0;
+  if (router_gemm_form(T, H, E, 1, MI_MOE_BF16, nullptr)) return router_gemm_form_bytes(T, E);
+  return router_ws_bytes(T, H, E);
 }
 
 // router_general.hip: fp32, 65 .. 256 experts, k up to 64
@@ -914,7 +931,22 @@ extern "C" int mi_moe_router_fused(const void* x, const void* gate_w, const floa
   if (!x || !gate_w || !gates_out || !idx_out) return MI_MOE_ENULL;
   if (!mi_aligned(x, 16) || !mi_aligned(gate_w, 16)) return MI_MOE_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (!streaming) return mi_router_general(x, gate_w, bias, T, H, E, k, dtype, logits_out, gates_out, idx_out, s);
+  if (!streaming) {
+    if (ws != nullptr && router_gemm_form(T, H, E, k, dtype, bias)) {
+      if (ws_bytes < router_gemm_form_bytes(T, E)) return MI_MOE_EWORKSPACE;
+      if (!mi_aligned(ws, 16)) return MI_MOE_EALIGN;
+      unsigned char* base = static_cast<unsigned char*>(ws);
+      int32_t* offsets = reinterpret_cast<int32_t*>(base + router_gemm_form_bytes(T, E) - 256);
+      void* logits = logits_out != nullptr ? logits_out : static_cast<void*>(base);
+      hipLaunchKernelGGL(router_one_expert_offsets_kernel, dim3(1), dim3(64), 0, s, offsets, T);
+      const int rc = mi_moe_scattered_gemm_ws(x, gate_w, logits, nullptr, offsets, T, H, E, 1, 1, 1, 1, dtype, -1, nullptr,
+                                              0, stream);
+      if (rc == MI_MOE_OK) return mi_moe_router_topk_softmax(logits, T, E, k, dtype, gates_out, idx_out, stream);
+      // a shape the tile kernels do not take (refused before anything of theirs was launched): the general kernel
+      if (rc != MI_MOE_EUNSUPPORTED && rc != MI_MOE_EALIGN) return rc;
+    }
+    return mi_router_general(x, gate_w, bias, T, H, E, k, dtype, logits_out, gates_out, idx_out, s);
+  }
   const size_t need = router_ws_bytes(T, H, E);
   if (ws != nullptr && need > 0) {  // few tokens and a workspace: K split across workgroups
     if (ws_bytes < need) return MI_MOE_EWORKSPACE;

@@ -121,7 +121,21 @@ __global__ __launch_bounds__(256) void router_general_kernel(const T* __restrict
     }
   }
   __syncthreads();
-  // top-k and softmax: wave w takes tokens 4 w .. 4 w + 3, lane l the experts l, l + 64, ...
+  // top-k and softmax: wave w takes tokens 4 w .. 4 w + 3 -- all four at once, 16 lanes per token, where k allows
+  // it, else one after the other with lane l on the experts l, l + 64, ...
+  if (k <= 16) {
+    const int row = wave * 4 + q;
+    const bool row_ok = tok0 + row < Trows;
+    float vals[NEB];
+#pragma unroll
+    for (int c = 0; c < NEB; ++c) {
+      const int e = r + c * 16;
+      vals[c] = e < E ? lg[row * EP + e] : 0.f;
+    }
+    const size_t trow = row_ok ? (size_t)(tok0 + row) : (size_t)(Trows - 1);
+    topk_softmax_row16<T, NEB>(vals, E, k, row_ok, gates + trow * k, idx + trow * k);
+    return;
+  }
   for (int i = 0; i < 4; ++i) {
     const int row = wave * 4 + i;
     if (tok0 + row >= Trows) break;  // (wave-uniform)

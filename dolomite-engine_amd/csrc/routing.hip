@@ -13,7 +13,7 @@
 // top-k softmax
 // ------------------------------------------------------------------------------------------------
 
-// One wavefront per row; lane l owns experts l, l + 64, ... (topk_row.h).
+// One wavefront per row; lane l owns experts l, l + 64, ... (topk_row.h): more than 256 experts or k > 16.
 template <typename T, int VPL>
 __global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__ logits, int Trows, int E, int k,
                                                            T* __restrict__ gates, int32_t* __restrict__ idx) {
@@ -30,11 +30,44 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__
   topk_softmax_row<T, VPL>(vals, E, k, gates + (size_t)row * k, idx + (size_t)row * k);
 }
 
+// Four rows per wavefront, 16 lanes per row (topk_row.h): up to 256 experts, k <= 16.  Lane j of a row's group
+// loads experts j, j + 16, ...: 16 consecutive values per load and row.
+template <typename T, int VPL>
+__global__ __launch_bounds__(256) void topk_softmax_rows16_kernel(const T* __restrict__ logits, int Trows, int E, int k,
+                                                                  T* __restrict__ gates, int32_t* __restrict__ idx) {
+  const int j16 = threadIdx.x & 15;
+  const int row = blockIdx.x * 16 + (threadIdx.x >> 4);
+  const bool row_ok = row < Trows;
+  const int rr = row_ok ? row : Trows - 1;  // surplus groups re-read the last row and write nothing
+  const T* src = logits + (size_t)rr * E;
+  float vals[VPL];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int e = j16 + i * 16;
+    vals[i] = e < E ? Elt<T>::load(src + e) : 0.f;
+  }
+  topk_softmax_row16<T, VPL>(vals, E, k, row_ok, gates + (size_t)rr * k, idx + (size_t)rr * k);
+}
+
 template <typename T>
 static int launch_topk(const void* logits, int T_, int E, int k, void* gates, int32_t* idx, hipStream_t s) {
   dim3 grid(mi_ceil_div(T_, 4)), block(256);
   const T* lg = static_cast<const T*>(logits);
   T* gt = static_cast<T*>(gates);
+  if (E <= 256 && k <= 16) {
+    dim3 grid16(mi_ceil_div(T_, 16));
+    if (E <= 16)
+      hipLaunchKernelGGL((topk_softmax_rows16_kernel<T, 1>), grid16, block, 0, s, lg, T_, E, k, gt, idx);
+    else if (E <= 32)
+      hipLaunchKernelGGL((topk_softmax_rows16_kernel<T, 2>), grid16, block, 0, s, lg, T_, E, k, gt, idx);
+    else if (E <= 64)
+      hipLaunchKernelGGL((topk_softmax_rows16_kernel<T, 4>), grid16, block, 0, s, lg, T_, E, k, gt, idx);
+    else if (E <= 128)
+      hipLaunchKernelGGL((topk_softmax_rows16_kernel<T, 8>), grid16, block, 0, s, lg, T_, E, k, gt, idx);
+    else
+      hipLaunchKernelGGL((topk_softmax_rows16_kernel<T, 16>), grid16, block, 0, s, lg, T_, E, k, gt, idx);
+    return mi_launch_status();
+  }
   if (E <= 64)
     hipLaunchKernelGGL((topk_softmax_kernel<T, 1>), grid, block, 0, s, lg, T_, E, k, gt, idx);
   else if (E <= 128)

@@ -157,6 +157,11 @@ def test_router_fused(device, dtype, T, H, E, k, bias):
     (torch.float16, 129, 1024, 256, 64, False),  # k beyond the streaming kernels' 8
     (torch.bfloat16, 50, 64, 40, 12, False),
     (torch.bfloat16, 2100, 48, 65, 2, False),
+    # many tokens, more than 64 experts, 16-bit: logits from the grouped GEMM's tile kernels, then the top-k kernel
+    (torch.bfloat16, 8200, 256, 128, 8, False),
+    (torch.float16, 4100, 512, 256, 6, False),
+    (torch.bfloat16, 10500, 48, 100, 20, False),   # (100 experts, hidden 48: not every tile kernel's shape)
+    (torch.bfloat16, 8200, 256, 128, 8, True),     # with a bias: the general kernel
 ])
 def test_router_general(device, dtype, T, H, E, k, bias):
     """fp32, more than 64 experts, k above 8: the general kernel behind the same entry point, held to the same
@@ -175,6 +180,10 @@ def test_router_general(device, dtype, T, H, E, k, bias):
     ref_logits = oracle.router_logits(x, w, b)
     tol = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.bfloat16: dict(rtol=1.6e-2, atol=1e-3),
            torch.float16: dict(rtol=2e-3, atol=1e-3)}[dtype]
+    if b is not None and dtype != torch.float32:
+        # (the product is rounded before the bias is added: where the two cancel, one rounding step of the product
+        # is large against the sum)
+        tol["atol"] += (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11) * float((ref_logits.float() - b).abs().max())
     torch.testing.assert_close(logits.float(), ref_logits.float(), **tol)
     vals, ref_idx = oracle.topk_canonical(logits, k)
     assert torch.equal(idx.cpu().long(), ref_idx)
