@@ -440,6 +440,47 @@ def measure_latency(m, x, reps=300):
     return out
 
 
+def measure_routing_stage(device, iters=30):
+    """The routing stage by itself at the workloads' shapes and at shapes with more experts: router (gate GEMM +
+    top-k + softmax), router + sort as the layer calls them, the stand-alone top-k + softmax on given logits, and
+    torch's linear + topk (no softmax, no sort) on the same inputs.  HIP events around back-to-back calls;
+    ``hbm_frac`` is the router's algorithmic bytes (x once, gate weights once, gates and indices out) over its time,
+    against the HBM peak."""
+    import torch
+    import torch.nn.functional as F
+
+    from dolomite_engine_amd import ops
+
+    shapes = [  # tokens, hidden, experts, k, dtype
+        (64, 4096, 64, 6, torch.bfloat16), (2048, 1536, 40, 8, torch.bfloat16), (16384, 1024, 32, 8, torch.bfloat16),
+        (32768, 1536, 40, 8, torch.bfloat16), (131072, 1536, 40, 8, torch.bfloat16),
+        (16384, 4096, 64, 6, torch.bfloat16), (4096, 2048, 128, 8, torch.bfloat16),
+        (32768, 2048, 128, 8, torch.bfloat16), (8192, 7168, 256, 8, torch.bfloat16),
+        (512, 256, 8, 2, torch.float32), (32768, 1536, 40, 8, torch.float32),
+    ]
+    g = torch.Generator(device="cpu").manual_seed(7)
+    rows = []
+    for T, H, E, k, dtype in shapes:
+        x = torch.randn(T, H, generator=g).to(dtype).to(device)
+        gw = (torch.randn(E, H, generator=g) * 0.02).to(dtype).to(device)
+        elt = x.element_size()
+        logits = F.linear(x, gw)
+        row = {"tokens": T, "hidden": H, "experts": E, "top_k": k, "dtype": str(dtype).replace("torch.", "")}
+        ms = _time_ms(lambda: ops.router_fused(x, gw, k), iters)
+        nbytes = T * H * elt + E * H * elt + T * k * (elt + 4)
+        row["router_us"] = ms * 1e3
+        row["router_hbm_frac"] = nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS
+        if ops.router_fused_sort_supported(x, E, k):
+            row["router_plus_sort_us"] = _time_ms(lambda: ops.router_fused_sort(x, gw, k), iters) * 1e3
+        else:
+            row["router_plus_sort_us"] = _time_ms(lambda: ops.sort_bin(ops.router_fused(x, gw, k)[2], E), iters) * 1e3
+        row["topk_softmax_us"] = _time_ms(lambda: ops.router_topk_softmax(logits, k), iters) * 1e3
+        row["torch_linear_topk_us"] = _time_ms(lambda: torch.topk(F.linear(x, gw), k), iters) * 1e3
+        rows.append(row)
+        del x, gw, logits
+    return rows
+
+
 def cpu_baseline(w, inputs, sample_tokens, iters=3):
     """Eager path of the oracle in fp32 on the host, on the first ``sample_tokens`` tokens."""
     import torch
@@ -510,6 +551,9 @@ def main():
                     help="also time a training step of the layer (forward + backward for the input and every "
                          "parameter, synthetic upstream gradient) through the kernel branch and through the eager "
                          "branch; reported as extra fields, value / ms_per_step stay the forward")
+    ap.add_argument("--routing", action="store_true",
+                    help="measure the routing stage alone (router, router + sort, top-k) at a list of shapes, "
+                         "print them as one JSON line and exit")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy so that a rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE run of this command contains a kernel of known traffic to scale by")
@@ -530,6 +574,11 @@ def main():
         sys.exit(1)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+
+    if args.routing:
+        print(json.dumps({"routing_stage": measure_routing_stage(device), "unit": "us per call, HIP events",
+                          "peak_hbm_gbs": PEAK_HBM_GBS}))
+        return
 
     w = oracle.WORKLOADS[args.workload]
     if args.tokens is not None:
