@@ -183,7 +183,8 @@ def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch
     # non-zero for few tokens (streaming kernels: K split over the chip) and for many tokens with more than 64
     # experts (16-bit: the logits come from the grouped GEMM's tile kernels, then the top-k kernel)
     ws_bytes = lib.mi_moe_router_fused_workspace_bytes(T, H, E) if (
-        split_k and (_router_streaming_supported(x, E, k) or (E > 64 and x.dtype != torch.float32))) else 0
+        split_k and (_router_streaming_supported(x, E, k)
+                     or (E > 64 and T * E >= 1 << 20 and x.dtype != torch.float32 and bias is None))) else 0
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
     with _stage("router_fused"):
         check(lib.mi_moe_router_fused(_ptr(x), _ptr(gate_weight), _ptr(bias), T, H, E, k, _code(x.dtype),
