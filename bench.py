@@ -706,6 +706,7 @@ def main():
         del m, x
         torch.cuda.empty_cache()
         out["workloads"] = {n: measure_compact(n, device) for n in oracle.WORKLOADS if n != w.name}
+        out["routing_stage"] = measure_routing_stage(device)
     if graph_ms is not None:
         out["ms_per_step_graph_replay"] = graph_ms
     if not args.no_cpu_baseline:
