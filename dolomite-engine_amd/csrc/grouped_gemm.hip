@@ -1775,8 +1775,14 @@ static int run_gemm(GemmArgs a, int dtype, bool glu, int cfg, int in_rows_bound,
   if (!tiled_aligned(a, elt)) return MI_MOE_EALIGN;
   if (dtype == MI_MOE_F32) {
     if (cfg < 0) {
+      // fp32 matrix instructions are slow enough that what matters is how many CUs have a tile.  Measured (up /
+      // down projection, us): 128 x 128 tiles beat 256 x 256 at every size tried (262144 rows, 40 experts, hidden
+      // 1536: 3240 / 1678 against 3359 / 1690; 65536 rows, 32 experts: 1136 / 585 against 1338 / 686), and below
+      // about two 128 x 128 tiles per CU the 32 x 256 tiles win (the reference's correctness configuration, 1024
+      // rows in 8 experts: 15 / 24 against 23 / 37; 4096 rows: 38 / 25 against 43 / 38 and, for 256 x 256, 73 / 127).
       const long avg = a.E > 0 ? (long)a.L / a.E : a.L;
-      cfg = avg >= 512 ? 0 : (avg >= 48 ? 1 : 5);
+      const long tiles128 = ((long)a.L / 128 + a.E / 2 + 1) * mi_ceil_div((glu ? 2 : 1) * a.N, 128);
+      cfg = avg < 48 ? 5 : ((avg >= 512 && tiles128 >= 512) ? 1 : 2);
     }
     return glu ? dispatch_cfg_f32<true>(a, cfg, s) : dispatch_cfg_f32<false>(a, cfg, s);
   }
