@@ -909,16 +909,23 @@ __global__ void router_one_expert_offsets_kernel(int32_t* offsets, int rows) {
   if (threadIdx.x == 0 && blockIdx.x == 0) offsets[0] = rows;
 }
 
+size_t mi_router_general_ws_bytes(int T_, int H, int E);  // router_general.hip
+
 extern "C" size_t mi_moe_router_fused_workspace_bytes(int T, int H, int E) {
   if (T < 0 || H < 1 || E < 1) return 0;
-  if (router_gemm_form(T, H, E, 1, MI_MOE_BF16, nullptr)) return router_gemm_form_bytes(T, E);
+  if (E > 64) {  // the general kernel's two forms that take a workspace: many tokens / few tokens
+    const size_t many = router_gemm_form(T, H, E, 1, MI_MOE_BF16, nullptr) ? router_gemm_form_bytes(T, E) : 0;
+    const size_t few = mi_router_general_ws_bytes(T, H, E);
+    return many > few ? many : few;
+  }
   return router_ws_bytes(T, H, E);
 }
 
 // router_general.hip: fp32, 65 .. 256 experts, k up to 64
 int mi_router_general_ok(int H, int E, int k, int dtype);
 int mi_router_general(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k, int dtype,
-                      void* logits_out, void* gates, int32_t* idx, hipStream_t s);
+                      void* logits_out, void* gates, int32_t* idx, void* ws, hipStream_t s);
+size_t mi_router_general_ws_bytes(int T_, int H, int E);
 
 extern "C" int mi_moe_router_fused(const void* x, const void* gate_w, const float* bias, int T, int H, int E, int k,
                                    int dtype, void* logits_out, void* gates_out, int32_t* idx_out, void* ws,
@@ -945,7 +952,13 @@ extern "C" int mi_moe_router_fused(const void* x, const void* gate_w, const floa
       // a shape the tile kernels do not take (refused before anything of theirs was launched): the general kernel
       if (rc != MI_MOE_EUNSUPPORTED && rc != MI_MOE_EALIGN) return rc;
     }
-    return mi_router_general(x, gate_w, bias, T, H, E, k, dtype, logits_out, gates_out, idx_out, s);
+    void* gws = nullptr;  // few tokens and more than 64 experts: the contraction cut into ranges
+    if (ws != nullptr && mi_router_general_ws_bytes(T, H, E) > 0) {
+      if (ws_bytes < mi_router_general_ws_bytes(T, H, E)) return MI_MOE_EWORKSPACE;
+      if (!mi_aligned(ws, 16)) return MI_MOE_EALIGN;
+      gws = ws;
+    }
+    return mi_router_general(x, gate_w, bias, T, H, E, k, dtype, logits_out, gates_out, idx_out, gws, s);
   }
   const size_t need = router_ws_bytes(T, H, E);
   if (ws != nullptr && need > 0) {  // few tokens and a workspace: K split across workgroups

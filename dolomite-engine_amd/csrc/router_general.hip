@@ -47,18 +47,75 @@ template <> struct GMfma<float> {
 #define ROUTER_GENERAL_MAX_E 256
 #define ROUTER_GENERAL_MAX_K 64
 
+// The tail both forms of the general kernel share.  Lane (r, q) of the wave that owns expert block eb holds the
+// fp32 sums of token r, experts 16 * eb + 4 * q + i: round to the model dtype, add the bias and round again, keep
+// the logit as fp32 in lg[token][expert] for the selection and write it out if the caller wants the logits.
+template <typename T, int EP>
+__device__ __forceinline__ void general_store_logits(const f32x4& sum, int eb, int r, int q, int tok0, int Trows, int E,
+                                                     const float* __restrict__ bias, float* __restrict__ lg,
+                                                     T* __restrict__ logits_out) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int e = eb * 16 + 4 * q + i;
+    float v = Elt<T>::round(sum[i]);
+    if (e < E) {
+      if (bias != nullptr) v = Elt<T>::round(v + bias[e]);
+      lg[r * EP + e] = v;
+      if (logits_out != nullptr && tok0 + r < Trows) Elt<T>::store(logits_out + (size_t)(tok0 + r) * E + e, v);
+    }
+  }
+}
+
+// top-k and softmax: wave w takes tokens 4 w .. 4 w + 3 -- all four at once, 16 lanes per token, where k allows
+// it, else one after the other with lane l on the experts l, l + 64, ...
+template <typename T, int NEB>
+__device__ __forceinline__ void general_topk(const float* __restrict__ lg, int wave, int r, int q, int tok0, int Trows,
+                                             int E, int k, T* __restrict__ gates, int32_t* __restrict__ idx) {
+  constexpr int EP = 16 * NEB;
+  constexpr int VPL = (NEB + 3) / 4;  // candidates per lane with one row per wave
+  if (k <= 16) {
+    const int row = wave * 4 + q;
+    const bool row_ok = tok0 + row < Trows;
+    float vals[NEB];
+#pragma unroll
+    for (int c = 0; c < NEB; ++c) {
+      const int e = r + c * 16;
+      vals[c] = e < E ? lg[row * EP + e] : 0.f;
+    }
+    const size_t trow = row_ok ? (size_t)(tok0 + row) : (size_t)(Trows - 1);
+    topk_softmax_row16<T, NEB>(vals, E, k, row_ok, gates + trow * k, idx + trow * k);
+    return;
+  }
+  const int lane = q * 16 + r;
+  for (int i = 0; i < 4; ++i) {
+    const int row = wave * 4 + i;
+    if (tok0 + row >= Trows) break;  // (wave-uniform)
+    float vals[VPL];
+#pragma unroll
+    for (int c = 0; c < VPL; ++c) {
+      const int e = lane + c * 64;
+      vals[c] = e < E ? lg[row * EP + e] : 0.f;
+    }
+    topk_softmax_row<T, VPL>(vals, E, k, gates + (size_t)(tok0 + row) * k, idx + (size_t)(tok0 + row) * k);
+  }
+}
+
 // NEB: expert blocks of 16 (E <= 16 * NEB).  LDS: [4 waves][NEB][64 lanes] partial accumulators, then
 // [16 tokens][16 * NEB] logits as fp32.
-template <typename T, int NEB>
+// SPLIT (few tokens, with the caller's workspace): blockIdx.y cuts the contraction into ranges of `steps_per_split`
+// steps; a workgroup adds up its range as below and writes the 16 x EP sums raw, [group][split][block][lane], and
+// router_general_finish_kernel adds a group's ranges in order and does the rest.  One workgroup per 16 tokens
+// alone leaves a decode batch on a handful of CUs, each pulling all gate weights through its four waves.
+template <typename T, int NEB, bool SPLIT>
 __global__ __launch_bounds__(256) void router_general_kernel(const T* __restrict__ x, const T* __restrict__ gw,
                                                              const float* __restrict__ bias, int Trows, int H, int E,
                                                              int k, T* __restrict__ logits_out, T* __restrict__ gates,
-                                                             int32_t* __restrict__ idx) {
+                                                             int32_t* __restrict__ idx, f32x4* __restrict__ partial,
+                                                             int steps_per_split) {
   constexpr int KSTEP = GMfma<T>::KSTEP;
   constexpr int LPL = KSTEP / 4;                   // elements per lane and step (two 16-byte loads)
   constexpr int HALF = LPL / 2;
   constexpr int EP = 16 * NEB;
-  constexpr int VPL = (NEB + 3) / 4;               // candidates per lane in the top-k
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   f32x4* red = reinterpret_cast<f32x4*>(smem_raw);                    // [4][NEB][64]
   float* lg = reinterpret_cast<float*>(smem_raw + 4 * NEB * 64 * 16);  // [16][EP]
@@ -73,7 +130,12 @@ __global__ __launch_bounds__(256) void router_general_kernel(const T* __restrict
 #pragma unroll
   for (int eb = 0; eb < NEB; ++eb) acc[eb] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const int neb = (E + 15) >> 4;
-  for (int k0 = wave * KSTEP; k0 < H; k0 += 4 * KSTEP) {
+  // wave w takes the steps first + w, first + w + 4, ... of the workgroup's range (all of them without SPLIT)
+  const int nsteps = (H + KSTEP - 1) / KSTEP;
+  const int first = SPLIT ? (int)blockIdx.y * steps_per_split : 0;
+  const int last = SPLIT ? (first + steps_per_split < nsteps ? first + steps_per_split : nsteps) : nsteps;
+  for (int st = first + wave; st < last; st += 4) {
+    const int k0 = st * KSTEP;
     const int kpos = k0 + q * LPL;
     const bool valid = kpos < H;  // the matrix instruction runs on all lanes: out-of-range k contributes zeros
     u32x4 xa[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
@@ -108,69 +170,113 @@ __global__ __launch_bounds__(256) void router_general_kernel(const T* __restrict
       f32x4 sum = red[eb * 64 + lane];
 #pragma unroll
       for (int w = 1; w < 4; ++w) sum += red[(w * NEB + eb) * 64 + lane];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int e = eb * 16 + 4 * q + i;
-        float v = Elt<T>::round(sum[i]);
-        if (e < E) {
-          if (bias != nullptr) v = Elt<T>::round(v + bias[e]);
-          lg[r * EP + e] = v;
-          if (logits_out != nullptr && tok0 + r < Trows) Elt<T>::store(logits_out + (size_t)(tok0 + r) * E + e, v);
-        }
+      if constexpr (SPLIT) {
+        partial[(((size_t)blockIdx.x * gridDim.y + blockIdx.y) * NEB + eb) * 64 + lane] = sum;
+      } else {
+        general_store_logits<T, EP>(sum, eb, r, q, tok0, Trows, E, bias, lg, logits_out);
       }
     }
   }
+  if constexpr (SPLIT) return;
   __syncthreads();
-  // top-k and softmax: wave w takes tokens 4 w .. 4 w + 3 -- all four at once, 16 lanes per token, where k allows
-  // it, else one after the other with lane l on the experts l, l + 64, ...
-  if (k <= 16) {
-    const int row = wave * 4 + q;
-    const bool row_ok = tok0 + row < Trows;
-    float vals[NEB];
+  general_topk<T, NEB>(lg, wave, r, q, tok0, Trows, E, k, gates, idx);
+}
+
+// Second launch of the SPLIT form: one workgroup per 16 tokens adds the ranges' sums in range order, then rounds,
+// adds the bias, writes the logits and selects exactly as the single launch does.
+template <typename T, int NEB>
+__global__ __launch_bounds__(256) void router_general_finish_kernel(const f32x4* __restrict__ partial, int splits,
+                                                                    const float* __restrict__ bias, int Trows, int E,
+                                                                    int k, T* __restrict__ logits_out,
+                                                                    T* __restrict__ gates, int32_t* __restrict__ idx) {
+  constexpr int EP = 16 * NEB;
+  __shared__ float lg[16 * EP];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int tok0 = blockIdx.x * 16;
+  const int neb = (E + 15) >> 4;
 #pragma unroll
-    for (int c = 0; c < NEB; ++c) {
-      const int e = r + c * 16;
-      vals[c] = e < E ? lg[row * EP + e] : 0.f;
-    }
-    const size_t trow = row_ok ? (size_t)(tok0 + row) : (size_t)(Trows - 1);
-    topk_softmax_row16<T, NEB>(vals, E, k, row_ok, gates + trow * k, idx + trow * k);
-    return;
-  }
-  for (int i = 0; i < 4; ++i) {
-    const int row = wave * 4 + i;
-    if (tok0 + row >= Trows) break;  // (wave-uniform)
-    float vals[VPL];
+  for (int eb0 = 0; eb0 < NEB; eb0 += 4) {
+    const int eb = eb0 + wave;
+    if (eb < NEB && eb < neb) {
+      const f32x4* src = partial + ((size_t)blockIdx.x * splits * NEB + eb) * 64 + lane;
+      // eight ranges' loads in flight at a time (the additions stay in range order)
+      f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+      for (int sp0 = 0; sp0 < splits; sp0 += 8) {
+        f32x4 v[8];
 #pragma unroll
-    for (int c = 0; c < VPL; ++c) {
-      const int e = lane + c * 64;
-      vals[c] = e < E ? lg[row * EP + e] : 0.f;
+        for (int j = 0; j < 8; ++j)
+          v[j] = sp0 + j < splits ? src[(size_t)(sp0 + j) * NEB * 64] : (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (sp0 + j < splits) sum += v[j];
+      }
+      general_store_logits<T, EP>(sum, eb, r, q, tok0, Trows, E, bias, lg, logits_out);
     }
-    topk_softmax_row<T, VPL>(vals, E, k, gates + (size_t)(tok0 + row) * k, idx + (size_t)(tok0 + row) * k);
   }
+  __syncthreads();
+  general_topk<T, NEB>(lg, wave, r, q, tok0, Trows, E, k, gates, idx);
+}
+
+// Ranges of the contraction for few tokens: enough workgroups for about two per CU, a step per wave at least.
+static int router_general_splits(int T_, int H, int dtype) {
+  const int kstep = dtype == MI_MOE_F32 ? 32 : 64;
+  const int nsteps = mi_ceil_div(H, kstep);
+  const int groups = mi_ceil_div(T_, 16);
+  int splits = mi_ceil_div(512, groups);
+  if (splits > nsteps / 4) splits = nsteps / 4;
+  return splits < 2 ? 1 : splits;
+}
+// partial sums of the SPLIT form: [group][split][block of 16 experts][lane] f32x4, for the most ranges any dtype takes
+size_t mi_router_general_ws_bytes(int T_, int H, int E) {
+  if (E <= 64) return 0;  // (up to 64 experts the general kernel serves fp32 and large k only: one launch)
+  const int splits = router_general_splits(T_, H, MI_MOE_F32);
+  if (splits < 2) return 0;
+  const int neb = E <= 128 ? 8 : 16;
+  return (size_t)mi_ceil_div(T_, 16) * splits * neb * 64 * sizeof(f32x4);
 }
 
 template <typename T, int NEB>
 static int launch_router_general(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
-                                 void* logits_out, void* gates, int32_t* idx, hipStream_t s) {
+                                 void* logits_out, void* gates, int32_t* idx, void* ws, int splits, hipStream_t s) {
   constexpr size_t lds = (size_t)4 * NEB * 64 * 16 + (size_t)16 * 16 * NEB * 4;
-  auto kern = router_general_kernel<T, NEB>;
+  const int groups = mi_ceil_div(T_, 16);
+  if (splits >= 2) {
+    auto kern = router_general_kernel<T, NEB, true>;
+    if (lds > 64 * 1024) {
+      static std::atomic<uint64_t> lds_ok{0};
+      const int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), (int)lds, lds_ok);
+      if (rc != MI_MOE_OK) return rc;
+    }
+    const int nsteps = mi_ceil_div(H, GMfma<T>::KSTEP);
+    const int sps = mi_ceil_div(nsteps, splits);
+    const int used = mi_ceil_div(nsteps, sps);  // every range has a step
+    hipLaunchKernelGGL(kern, dim3(groups, used), dim3(256), lds, s, static_cast<const T*>(x), static_cast<const T*>(gw),
+                       bias, T_, H, E, k, static_cast<T*>(logits_out), static_cast<T*>(gates), idx,
+                       static_cast<f32x4*>(ws), sps);
+    hipLaunchKernelGGL((router_general_finish_kernel<T, NEB>), dim3(groups), dim3(256), 0, s,
+                       static_cast<const f32x4*>(ws), used, bias, T_, E, k, static_cast<T*>(logits_out),
+                       static_cast<T*>(gates), idx);
+    return mi_launch_status();
+  }
+  auto kern = router_general_kernel<T, NEB, false>;
   if (lds > 64 * 1024) {
     static std::atomic<uint64_t> lds_ok{0};
     const int rc = mi_allow_lds_once(reinterpret_cast<const void*>(kern), (int)lds, lds_ok);
     if (rc != MI_MOE_OK) return rc;
   }
-  hipLaunchKernelGGL(kern, dim3(mi_ceil_div(T_, 16)), dim3(256), lds, s, static_cast<const T*>(x),
+  hipLaunchKernelGGL(kern, dim3(groups), dim3(256), lds, s, static_cast<const T*>(x),
                      static_cast<const T*>(gw), bias, T_, H, E, k, static_cast<T*>(logits_out),
-                     static_cast<T*>(gates), idx);
+                     static_cast<T*>(gates), idx, static_cast<f32x4*>(nullptr), 0);
   return mi_launch_status();
 }
 
 template <typename T>
 static int router_general_by_blocks(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k,
-                                    void* logits_out, void* gates, int32_t* idx, hipStream_t s) {
-  if (E <= 64) return launch_router_general<T, 4>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, s);
-  if (E <= 128) return launch_router_general<T, 8>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, s);
-  return launch_router_general<T, 16>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, s);
+                                    void* logits_out, void* gates, int32_t* idx, void* ws, int splits, hipStream_t s) {
+  if (E <= 64) return launch_router_general<T, 4>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, ws, splits, s);
+  if (E <= 128) return launch_router_general<T, 8>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, ws, splits, s);
+  return launch_router_general<T, 16>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, ws, splits, s);
 }
 
 // Shapes the general kernel takes: whole 16-byte pieces per lane and step.
@@ -181,13 +287,18 @@ int mi_router_general_ok(int H, int E, int k, int dtype) {
 }
 
 // Called by mi_moe_router_fused (router_fused.hip) for what its streaming kernels do not take; arguments are
-// validated there.
+// validated there.  `ws` (or null) holds mi_router_general_ws_bytes(T, H, E) bytes: with more than 64 experts and
+// few tokens the contraction is then cut into ranges over many workgroups.
 int mi_router_general(const void* x, const void* gw, const float* bias, int T_, int H, int E, int k, int dtype,
-                      void* logits_out, void* gates, int32_t* idx, hipStream_t s) {
+                      void* logits_out, void* gates, int32_t* idx, void* ws, hipStream_t s) {
+  const int splits = (ws != nullptr && E > 64) ? router_general_splits(T_, H, dtype) : 1;
   switch (dtype) {
-    case MI_MOE_F32: return router_general_by_blocks<float>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, s);
-    case MI_MOE_F16: return router_general_by_blocks<f16_t>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, s);
-    case MI_MOE_BF16: return router_general_by_blocks<bf16_t>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, s);
+    case MI_MOE_F32:
+      return router_general_by_blocks<float>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, ws, splits, s);
+    case MI_MOE_F16:
+      return router_general_by_blocks<f16_t>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, ws, splits, s);
+    case MI_MOE_BF16:
+      return router_general_by_blocks<bf16_t>(x, gw, bias, T_, H, E, k, logits_out, gates, idx, ws, splits, s);
     default: return MI_MOE_EDTYPE;
   }
 }

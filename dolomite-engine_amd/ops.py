@@ -180,11 +180,10 @@ def router_fused(x: torch.Tensor, gate_weight: torch.Tensor, k: int, bias: torch
     gates = torch.empty((T, k), dtype=x.dtype, device=x.device)
     idx = torch.empty((T, k), dtype=torch.int32, device=x.device)
     lib = _lib.load()
-    # non-zero for few tokens (streaming kernels: K split over the chip) and for many tokens with more than 64
-    # experts (16-bit: the logits come from the grouped GEMM's tile kernels, then the top-k kernel)
+    # non-zero for few tokens (K split over the chip) and, with more than 64 experts, for many tokens (16-bit: the
+    # logits come from the grouped GEMM's tile kernels, then the top-k kernel)
     ws_bytes = lib.mi_moe_router_fused_workspace_bytes(T, H, E) if (
-        split_k and (_router_streaming_supported(x, E, k)
-                     or (E > 64 and T * E >= 1 << 20 and x.dtype != torch.float32 and bias is None))) else 0
+        split_k and (_router_streaming_supported(x, E, k) or E > 64)) else 0
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
     with _stage("router_fused"):
         check(lib.mi_moe_router_fused(_ptr(x), _ptr(gate_weight), _ptr(bias), T, H, E, k, _code(x.dtype),

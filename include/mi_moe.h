@@ -81,7 +81,9 @@ int mi_moe_router_topk_softmax(const void* logits, int T, int E, int k, int dtyp
  *                  mi_moe_router_fused_workspace_bytes(T, H, E) bytes (non-zero for T <= 1024) the
  *                  contraction is split over many workgroups and finished by a second small launch -- a few
  *                  tokens alone cannot keep more than T/16 compute units busy; with NULL one launch does it all.
- *                  The size is also non-zero for more than 64 experts with T * E >= 2^20: F16 / BF16 without a
+ *                  More than 64 experts: non-zero for few tokens too (the general kernel then cuts the
+ *                  contraction into ranges over many workgroups and a second launch adds them in order), and
+ *                  for T * E >= 2^20: F16 / BF16 without a
  *                  bias then take their logits from the grouped GEMM's tile kernels (one expert that owns every
  *                  row; the logits go to logits_out or, without one, into the workspace) and run the top-k
  *                  kernel on them -- the general kernel re-reads the gate weights for every 16 tokens.

@@ -162,6 +162,11 @@ def test_router_fused(device, dtype, T, H, E, k, bias):
     (torch.float16, 4100, 512, 256, 6, False),
     (torch.bfloat16, 10500, 48, 100, 20, False),   # (100 experts, hidden 48: not every tile kernel's shape)
     (torch.bfloat16, 8200, 256, 128, 8, True),     # with a bias: the general kernel
+    # few tokens, more than 64 experts: the contraction cut into ranges over many workgroups
+    (torch.bfloat16, 64, 7168, 256, 8, False),
+    (torch.float16, 1, 2048, 128, 8, True),
+    (torch.bfloat16, 1000, 2064, 200, 20, True),
+    (torch.float32, 33, 4096, 130, 6, False),
 ])
 def test_router_general(device, dtype, T, H, E, k, bias):
     """fp32, more than 64 experts, k above 8: the general kernel behind the same entry point, held to the same
@@ -194,6 +199,17 @@ def test_router_general(device, dtype, T, H, E, k, bias):
         assert (gates.cpu().view(torch.int16).int() - ref_gates.view(torch.int16).int()).abs().max() <= 1
     _, gates2, idx2 = ops.router_fused(x.to(device), w.to(device), k, bias=bd)
     assert torch.equal(idx2, idx) and torch.equal(gates2, gates)
+    # without a workspace (one launch; few tokens with many experts, and many tokens, take other forms with one):
+    # another summation order, the same contract on its own logits
+    logits3, gates3, idx3 = ops.router_fused(x.to(device), w.to(device), k, bias=bd, return_logits=True, split_k=False)
+    torch.testing.assert_close(logits3.cpu().float(), ref_logits.float(), **tol)
+    vals3, ref_idx3 = oracle.topk_canonical(logits3.cpu(), k)
+    assert torch.equal(idx3.cpu().long(), ref_idx3)
+    ref_gates3 = oracle.softmax_topk(vals3, dtype)
+    if dtype == torch.float32:
+        torch.testing.assert_close(gates3.cpu(), ref_gates3, rtol=1e-5, atol=1e-7)
+    else:
+        assert (gates3.cpu().view(torch.int16).int() - ref_gates3.view(torch.int16).int()).abs().max() <= 1
 
 
 def test_router_general_ties_and_special_values(device):
