@@ -454,7 +454,8 @@ def measure_routing_stage(device, iters=30):
     shapes = [  # tokens, hidden, experts, k, dtype
         (64, 4096, 64, 6, torch.bfloat16), (2048, 1536, 40, 8, torch.bfloat16), (16384, 1024, 32, 8, torch.bfloat16),
         (32768, 1536, 40, 8, torch.bfloat16), (131072, 1536, 40, 8, torch.bfloat16),
-        (16384, 4096, 64, 6, torch.bfloat16), (4096, 2048, 128, 8, torch.bfloat16),
+        (16384, 4096, 64, 6, torch.bfloat16), (64, 4096, 128, 8, torch.bfloat16), (64, 7168, 256, 8, torch.bfloat16),
+        (4096, 2048, 128, 8, torch.bfloat16),
         (32768, 2048, 128, 8, torch.bfloat16), (8192, 7168, 256, 8, torch.bfloat16),
         (512, 256, 8, 2, torch.float32), (32768, 1536, 40, 8, torch.float32),
     ]
