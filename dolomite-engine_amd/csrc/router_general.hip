@@ -222,6 +222,7 @@ __global__ __launch_bounds__(256) void router_general_finish_kernel(const f32x4*
 static int router_general_splits(int T_, int H, int dtype) {
   const int kstep = dtype == MI_MOE_F32 ? 32 : 64;
   const int nsteps = mi_ceil_div(H, kstep);
+  if (T_ < 1) return 1;
   const int groups = mi_ceil_div(T_, 16);
   int splits = mi_ceil_div(512, groups);
   if (splits > nsteps / 4) splits = nsteps / 4;

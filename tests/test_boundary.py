@@ -86,6 +86,13 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_router_fused_workspace_bytes(321, 1536, 40) == 0
     assert lib.mi_moe_router_fused_workspace_bytes(1024, 4096, 64) > 0
     assert lib.mi_moe_router_fused_workspace_bytes(1025, 4096, 64) == 0
+    # more than 64 experts: few tokens (the contraction in ranges: groups x ranges x expert blocks x 1 KiB of
+    # partial sums, up to 511 groups of 16 tokens), many tokens (T x E >= 2^20: T x E 16-bit logits + 256 bytes),
+    # nothing where neither applies; an empty batch needs none
+    assert lib.mi_moe_router_fused_workspace_bytes(64, 4096, 128) == 4 * 32 * 8 * 1024
+    assert lib.mi_moe_router_fused_workspace_bytes(32768, 2048, 128) == 32768 * 128 * 2 + 256
+    assert lib.mi_moe_router_fused_workspace_bytes(8192, 2048, 65) == 0
+    assert lib.mi_moe_router_fused_workspace_bytes(0, 4096, 128) == 0
     assert lib.mi_moe_router_fused_sort_workspace_bytes(64, 4096, 64, 6) == lib.mi_moe_router_fused_workspace_bytes(64, 4096, 64) + 256
     assert lib.mi_moe_router_fused_sort_workspace_bytes(2048, 4096, 64, 8) == 0   # many tokens, gate weights beyond LDS
     assert lib.mi_moe_router_fused_sort_workspace_bytes(1024, 1024, 64, 9) == 0   # T * k beyond the one-block sort
