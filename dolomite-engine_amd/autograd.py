@@ -215,20 +215,28 @@ class FusedRouter(torch.autograd.Function):
 
         logits = x @ gate_w^T (+ bias) in x.dtype;  experts = top-k;  gates = softmax over the k picked logits
 
-    Returns (logits, gates, experts).  The backward takes the gradients that arrive at ``gates`` (from the expert
-    combine) and at ``logits`` (from the auxiliary loss), forms d logits in one element-wise kernel and runs the two
-    products d x = d logits @ gate_w and d gate_w = d logits^T @ x on the grouped GEMM / grouped weight-gradient
-    kernels as one expert that owns every token: no library GEMM in either direction."""
+    Returns (logits, gates, experts, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets); the last three are
+    the expert sort of the selection where the router kernel can fold it in (ops.router_fused_sort: its first pass
+    is the router's epilogue), else None and the caller sorts.  The backward takes the gradients that arrive at
+    ``gates`` (from the expert combine) and at ``logits`` (from the auxiliary loss), forms d logits in one
+    element-wise kernel and runs the two products d x = d logits @ gate_w and d gate_w = d logits^T @ x on the
+    grouped GEMM / grouped weight-gradient kernels as one expert that owns every token: no library GEMM in either
+    direction."""
 
     @staticmethod
     def forward(ctx, x, gate_w, bias, k):
-        logits, gates, experts = ops.router_fused(x, gate_w, k, bias=bias, return_logits=True)
+        se = ss = off = None
+        if ops.router_fused_sort_supported(x, gate_w.shape[0], k):
+            logits, gates, experts, se, ss, off = ops.router_fused_sort(x, gate_w, k, bias=bias, return_logits=True)
+            ctx.mark_non_differentiable(experts, se, ss, off)
+        else:
+            logits, gates, experts = ops.router_fused(x, gate_w, k, bias=bias, return_logits=True)
+            ctx.mark_non_differentiable(experts)
         ctx.save_for_backward(x, gate_w, logits, experts)
-        ctx.mark_non_differentiable(experts)
-        return logits, gates, experts
+        return logits, gates, experts, se, ss, off
 
     @staticmethod
-    def backward(ctx, d_logits, d_gates, _):
+    def backward(ctx, d_logits, d_gates, *_):
         x, gate_w, logits, experts = ctx.saved_tensors
         T, H = x.shape
         if d_logits is None and d_gates is None:

@@ -260,9 +260,10 @@ class MoE(nn.Module):
             else:
                 hidden_states = F.rms_norm(hidden_states, (self.hidden_size,), norm_weight, norm_eps)
 
-        router_logits, router_weights, selected_experts = (
-            routed if routed is not None else self._compute_routing_weights(hidden_states)
-        )
+        if routed is None:
+            # (with a gradient the router function may hand back the expert sort as well)
+            *routed, presorted = self._route(hidden_states)
+        router_logits, router_weights, selected_experts = routed
 
         # the tail can only be folded in where nothing sits between the expert sum and it
         fuse_tail = (
@@ -324,15 +325,23 @@ class MoE(nn.Module):
         )
 
     def _compute_routing_weights(self, hidden_states: torch.Tensor):
-        """moe.py:246-257.  On the kernel path the gate GEMM, top-k and softmax are one kernel in every dtype; in
-        eval mode the (T, E) logits are never written (only the training aux loss and the backward read them); with
-        a gradient the same kernel runs inside autograd.FusedRouter, whose backward is kernels too."""
+        """moe.py:246-257: (router_logits, router_weights, selected_experts)."""
+        return self._route(hidden_states)[:3]
+
+    def _route(self, hidden_states: torch.Tensor):
+        """moe.py:246-257, plus the expert sort where the router produced it: (router_logits, router_weights,
+        selected_experts, presorted or None).  On the kernel path the gate GEMM, top-k and softmax are one kernel in
+        every dtype; in eval mode the (T, E) logits are never written (only the training aux loss and the backward
+        read them); with a gradient the same kernel runs inside autograd.FusedRouter, whose backward is kernels
+        too."""
         if (is_kernel_allowed(Kernel.scattermoe) and hidden_states.is_cuda
                 and ops.router_fused_supported(hidden_states, self.num_experts, self.top_k)):
             if self._needs_grad(hidden_states):
-                return FusedRouter.apply(hidden_states, self.gate.weight, self.router_logit_bias, self.top_k)
-            return ops.router_fused(hidden_states, self.gate.weight, self.top_k, bias=self.router_logit_bias,
-                                    return_logits=self.training)
+                logits, weights, experts, *srt = FusedRouter.apply(hidden_states, self.gate.weight,
+                                                                   self.router_logit_bias, self.top_k)
+                return logits, weights, experts, (srt if srt[0] is not None else None)
+            return (*ops.router_fused(hidden_states, self.gate.weight, self.top_k, bias=self.router_logit_bias,
+                                      return_logits=self.training), None)
 
         router_logits = self.gate(hidden_states)
         if self.router_logit_bias is not None:
@@ -358,7 +367,7 @@ class MoE(nn.Module):
             router_weights = F.softmax(router_weights.float(), dim=-1)
             router_weights = router_weights.type_as(hidden_states)
 
-        return router_logits, router_weights, selected_experts
+        return router_logits, router_weights, selected_experts, None
 
     def _compute_experts(self, hidden_states: torch.Tensor, router_weights: torch.Tensor,
                          selected_experts: torch.Tensor, tail: tuple | None = None,

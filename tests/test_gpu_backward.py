@@ -394,8 +394,15 @@ def test_fused_router_function(device, dtype, T, H, E, k):
     print(f"FusedRouter {dtype} T={T} H={H} E={E} k={k}", flush=True)
 
     x, w = x0.clone().requires_grad_(True), w0.clone().requires_grad_(True)
-    logits, gates, experts = FusedRouter.apply(x, w, None, k)
+    logits, gates, experts, *srt = FusedRouter.apply(x, w, None, k)
     ((gates * dg).sum() + (logits * dl).sum()).backward()
+    from dolomite_engine_amd import ops
+
+    # where the router kernel folds the expert sort in, the function hands it back: the sort of its selection
+    assert (srt[0] is not None) == ops.router_fused_sort_supported(x0, E, k)
+    if srt[0] is not None:
+        for got, want in zip(srt, ops.sort_bin(experts, E)):
+            assert torch.equal(got, want)
 
     xr, wr = x0.clone().requires_grad_(True), w0.clone().requires_grad_(True)
     logits_r = torch.nn.functional.linear(xr, wr)
