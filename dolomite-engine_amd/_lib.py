@@ -57,6 +57,7 @@ SIGNATURES: dict[str, tuple] = {
     "mi_moe_combine_grad_gates": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mi_moe_grouped_wgrad_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mi_moe_grouped_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "mi_moe_grouped_wgrad_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mi_moe_grouped_wgrad_naive": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "mi_moe_aux_loss_workspace_bytes": (_sz, [_i, _i]),
     "mi_moe_aux_loss": (_i, [_vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _vp]),

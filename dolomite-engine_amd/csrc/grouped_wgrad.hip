@@ -602,6 +602,118 @@ extern "C" int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const v
   return mi_launch_status();
 }
 
+// ---- fp32 weight gradient on the matrix cores ----------------------------------------------------------------
+// One workgroup per (expert, 128 x 128 tile of dW) walks the expert's rows 16 at a time: both operand slices go
+// global -> registers -> LDS exactly as they lie in memory ([row][column], the loads of the next slice in flight
+// while this one is multiplied), and the fragments of v_mfma_f32_32x32x2f32 are single floats -- lane l supplies
+// a[row 2 j + l / 32][column l % 32] and the same element of b -- so no transposing read is needed: 32 lanes read
+// 32 consecutive floats of one slice row.  The row pitch of 160 floats puts the two half waves (rows 2 j and
+// 2 j + 1) on different halves of the 64 banks.  The rows are added in ascending order by one workgroup:
+// deterministic, no workspace; experts without rows get zeros.  M % 4 == N % 4 == 0.
+#define WGRAD_F32_TILE 128
+#define WGRAD_F32_ROWS 16
+#define WGRAD_F32_PITCH 160
+__global__ __launch_bounds__(256) void grouped_wgrad_f32_kernel(const float* __restrict__ a,
+                                                                const int32_t* __restrict__ a_idx,
+                                                                const float* __restrict__ b,
+                                                                const int32_t* __restrict__ b_idx,
+                                                                const int32_t* __restrict__ offsets,
+                                                                float* __restrict__ dw, int M, int N) {
+  constexpr int TILE = WGRAD_F32_TILE, RS = WGRAD_F32_ROWS, PITCH = WGRAD_F32_PITCH;
+  __shared__ __attribute__((aligned(16))) float sa[2][RS * PITCH];
+  __shared__ __attribute__((aligned(16))) float sb[2][RS * PITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int e = blockIdx.z;
+  const int m0 = blockIdx.y * TILE, n0 = blockIdx.x * TILE;
+  const int begin = e > 0 ? offsets[e - 1] : 0, end = offsets[e];
+  const int nslices = (end - begin + RS - 1) / RS;
+
+  // staging: thread t takes the float4 at column 4 (t % 32) of the slice rows t / 32 and t / 32 + 8, of both operands
+  const int lrow = tid >> 5, lcol = (tid & 31) * 4;
+  f32x4 ra[2], rb[2];
+  auto load_slice = [&](int sl) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int r = begin + sl * RS + lrow + 8 * j;
+      ra[j] = rb[j] = (f32x4){0.f, 0.f, 0.f, 0.f};  // rows past the expert's end and columns past the edge add nothing
+      if (r < end) {
+        const size_t ar = a_idx ? (size_t)a_idx[r] : (size_t)r;
+        const size_t br = b_idx ? (size_t)b_idx[r] : (size_t)r;
+        if (m0 + lcol < M) ra[j] = *reinterpret_cast<const f32x4*>(a + ar * M + m0 + lcol);
+        if (n0 + lcol < N) rb[j] = *reinterpret_cast<const f32x4*>(b + br * N + n0 + lcol);
+      }
+    }
+  };
+  auto store_slice = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      *reinterpret_cast<f32x4*>(&sa[buf][(lrow + 8 * j) * PITCH + lcol]) = ra[j];
+      *reinterpret_cast<f32x4*>(&sb[buf][(lrow + 8 * j) * PITCH + lcol]) = rb[j];
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
+
+  const int fcol = lane & 31, fk = lane >> 5;
+  if (nslices > 0) {
+    load_slice(0);
+    store_slice(0);
+  }
+  __syncthreads();
+  for (int sl = 0; sl < nslices; ++sl) {
+    const int buf = sl & 1;
+    if (sl + 1 < nslices) load_slice(sl + 1);
+#pragma unroll
+    for (int j = 0; j < RS / 2; ++j) {
+      const float* pa = &sa[buf][(2 * j + fk) * PITCH + wm * 64 + fcol];
+      const float* pb = &sb[buf][(2 * j + fk) * PITCH + wn * 64 + fcol];
+      const float af[2] = {pa[0], pa[32]}, bf[2] = {pb[0], pb[32]};
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+          acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mb], bf[nb], acc[mb][nb], 0, 0, 0);
+    }
+    if (sl + 1 < nslices) store_slice(buf ^ 1);
+    __syncthreads();
+  }
+  // register i of lane l: row 8 (i / 4) + 4 (l / 32) + i % 4 of the block (the a operand's index), column l % 32
+  float* __restrict__ out = dw + (size_t)e * M * N;
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const int n = n0 + wn * 64 + nb * 32 + fcol;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = m0 + wm * 64 + mb * 32 + 8 * (i / 4) + 4 * fk + (i % 4);
+        if (m < M && n < N) out[(size_t)m * N + n] = acc[mb][nb][i];
+      }
+    }
+}
+
+extern "C" int mi_moe_grouped_wgrad_f32(const float* a, const int32_t* a_idx, const float* b, const int32_t* b_idx,
+                                        const int32_t* expert_offsets, float* dw, int L, int M, int N, int E,
+                                        mi_moe_stream_t stream) {
+  if (L < 0 || M < 1 || N < 1 || E < 1 || E > 65535) return MI_MOE_ESHAPE;
+  if (M % 4 != 0 || N % 4 != 0) return MI_MOE_EUNSUPPORTED;
+  if (!dw || !expert_offsets) return MI_MOE_ENULL;
+  if (L > 0 && (!a || !b)) return MI_MOE_ENULL;
+  if (!mi_aligned(a, 16) || !mi_aligned(b, 16)) return MI_MOE_EALIGN;
+  const dim3 grid(mi_ceil_div(N, WGRAD_F32_TILE), mi_ceil_div(M, WGRAD_F32_TILE), E);
+  if (grid.y > 65535u) return MI_MOE_ESHAPE;
+  hipLaunchKernelGGL(grouped_wgrad_f32_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a, a_idx, b, b_idx,
+                     expert_offsets, dw, M, N);
+  return mi_launch_status();
+}
+
 // ---- any-shape / any-dtype weight gradient (one thread per element of dW) ------------------------------------
 // For fp32 and for shapes the matrix-core kernel above does not take.  Every element sums its expert's rows in
 // ascending order in fp32 (deterministic) and is rounded once.  Correct, not fast; no workspace, no host round trip.

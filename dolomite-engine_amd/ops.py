@@ -559,8 +559,8 @@ def grouped_wgrad(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor
 
     ``a`` (rows_a, M) and ``b`` (rows_b, N); ``a_idx`` / ``b_idx`` (L,) int32 map a sorted row to a row of the
     operand (``None``: the operand is already in sorted order and has L rows).  The per-expert weight gradient of
-    the backward of ``scattered_experts`` (moe.py:91-101).  16-bit operands with M % 8 == N % 8 == 0 run on the
-    matrix cores; fp32 and other shapes on a one-thread-per-element kernel."""
+    the backward of ``scattered_experts`` (moe.py:91-101).  16-bit operands with M % 8 == N % 8 == 0 and fp32 operands
+    with M % 4 == N % 4 == 0 run on the matrix cores; other shapes on a one-thread-per-element kernel."""
     _dev(a, b, expert_offsets, a_idx, b_idx)
     _no_grad(a, b)
     a = a.contiguous()
@@ -581,9 +581,16 @@ def grouped_wgrad(a: torch.Tensor, b: torch.Tensor, expert_offsets: torch.Tensor
     b_idx = None if b_idx is None else b_idx.contiguous()
     expert_offsets = _i32(expert_offsets).contiguous()
     lib = _lib.load()
+    if a.dtype == torch.float32 and M % 4 == 0 and N % 4 == 0 and E <= 65535:
+        # fp32 on its own matrix instruction: one workgroup per (expert, tile) adds the rows in order, no workspace
+        dw = torch.empty((E, M, N), dtype=a.dtype, device=a.device)
+        with _stage("grouped_wgrad"):
+            check(lib.mi_moe_grouped_wgrad_f32(_ptr(a), _ptr(a_idx), _ptr(b), _ptr(b_idx), _ptr(expert_offsets), _ptr(dw),
+                                               L, M, N, E, _stream()))
+        return dw
     if not grouped_wgrad_supported(a, b, E):
-        # fp32 (no matrix-core path for it) and odd shapes: the one-thread-per-element kernel, on the device like
-        # everything else (no per-expert host loop, no synchronisation)
+        # odd shapes: the one-thread-per-element kernel, on the device like everything else (no per-expert host
+        # loop, no synchronisation)
         if a.dtype != torch.float32:
             _warn_once("slow_wgrad", f"grouped weight gradient with M={M}, N={N}, E={E}, {a.dtype}: running the slow "
                        "one-thread-per-element kernel (the matrix-core kernel needs M % 8 == N % 8 == 0, E <= 256)")

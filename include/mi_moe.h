@@ -341,6 +341,13 @@ int mi_moe_grouped_wgrad(const void* a, const int32_t* a_idx, const void* b, con
                          const int32_t* expert_offsets, void* dw, void* workspace, size_t workspace_bytes,
                          int L, int a_rows, int b_rows, int M, int N, int E, int dtype, mi_moe_stream_t stream);
 
+/* The same sums for F32 operands on the fp32 matrix instruction (no counterpart of its own in the reference: its
+ * scattermoe backward serves every dtype): one workgroup per (expert, 128 x 128 tile of dw) adds the expert's rows
+ * in ascending order -- deterministic, no workspace.  M % 4 == 0, N % 4 == 0, 16-byte aligned operands, E <= 65535. */
+int mi_moe_grouped_wgrad_f32(const float* a, const int32_t* a_idx, const float* b, const int32_t* b_idx,
+                             const int32_t* expert_offsets, float* dw, int L, int M, int N, int E,
+                             mi_moe_stream_t stream);
+
 /* The same sums for any shape and for F32 as well (the matrix-core kernel above takes 16-bit operands with
  * M % 8 == N % 8 == 0 only): one thread per element of dw, the expert's rows added in ascending order in fp32, one
  * rounding.  Slow; no workspace.  M <= 262140, E <= 65535. */

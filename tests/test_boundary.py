@@ -121,6 +121,9 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mi_moe_probe_kloop(0, None, 4 << 20, 10, None, 0, None) == E_NULL
     assert lib.mi_moe_swiglu_forward(None, None, 4, 16, _lib.BF16, None) == E_NULL
     assert lib.mi_moe_swiglu_forward(None, None, 0, 16, _lib.BF16, None) == 0
+    assert lib.mi_moe_grouped_wgrad_f32(None, None, None, None, None, None, 16, 8, 8, 0, None) == E_SHAPE
+    assert lib.mi_moe_grouped_wgrad_f32(None, None, None, None, None, None, 16, 6, 8, 4, None) == E_UNSUP
+    assert lib.mi_moe_grouped_wgrad_f32(None, None, None, None, None, None, 16, 8, 8, 4, None) == E_NULL
     assert lib.mi_moe_grouped_wgrad_naive(None, None, None, None, None, None, 16, 8, 8, 4, 7, None) == E_DTYPE
     assert lib.mi_moe_grouped_wgrad_naive(None, None, None, None, None, None, 16, 8, 8, 4, _lib.F32, None) == E_NULL
     # 16-bit problems the matrix-core kernels cannot take are refused, not run on the slow kernel behind the

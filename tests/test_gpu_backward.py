@@ -144,8 +144,8 @@ def _seeded_counts(L, weights, g):
     return torch.bincount(draws, minlength=weights.numel())
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("L,E,M,N,rows_other", WGRAD_CASES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("L,E,M,N,rows_other", WGRAD_CASES + [(900, 6, 132, 260, 100)])  # (fp32: multiples of 4)
 @pytest.mark.parametrize("gather", ["a", "b", "none", "both"])
 def test_grouped_wgrad(device, dtype, L, E, M, N, rows_other, gather):
     g = torch.Generator().manual_seed(L * 7 + E)
@@ -167,7 +167,7 @@ def test_grouped_wgrad(device, dtype, L, E, M, N, rows_other, gather):
                                None if a_idx is None else a_idx.to(device), None if b_idx is None else b_idx.to(device))
     assert got.dtype == dtype and tuple(got.shape) == (E, M, N)
     ref = _wgrad_reference(a, b, offsets, a_idx, b_idx)
-    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -20}[dtype]
     # fp32 accumulation of up to L products of unit-variance terms, one rounding to the dtype
     torch.testing.assert_close(got.cpu().double(), ref, rtol=2 * eps, atol=2e-5 * max(1.0, counts.max().item()) ** 0.5 + 1e-6)
     # experts without rows get exact zeros
