@@ -106,7 +106,10 @@ def test_layer_fp8_sizes_not_multiples_of_16(device, H, I):
     against the oracle."""
     import dataclasses
 
+    from dolomite_engine_amd import ops
+
     w = dataclasses.replace(oracle.WORKLOADS["decode-fp8"], E=8, k=2, H=H, I=I, name="fp8-odd-sizes")
+    ops._WARNED.discard(("fp8_widened", H, I))  # (the warning is given once per process and shape)
     with pytest.warns(RuntimeWarning, match="multiples of 16"):
         _check_layer(w, 300, device, dict(rtol=2e-2, atol=2e-2))
 
