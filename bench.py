@@ -482,8 +482,9 @@ def measure_routing_stage(device, iters=30):
     return rows
 
 
-def cpu_baseline(w, inputs, sample_tokens, iters=3):
-    """Eager path of the oracle in fp32 on the host, on the first ``sample_tokens`` tokens."""
+def cpu_baseline(w, inputs, sample_tokens, budget_s=10.0):
+    """Eager path of the oracle in fp32 on the host, on the first ``sample_tokens`` tokens: one warm-up, then as
+    many timed forwards as fit ``budget_s`` seconds (2 to 8), median."""
     import torch
 
     from oracle import moe_oracle as oracle
@@ -503,7 +504,9 @@ def cpu_baseline(w, inputs, sample_tokens, iters=3):
         _, gates, idx = oracle.route(x, gate_w, w.k, bias=bias)
         return oracle.experts_eager(x, gates, idx, w_fc, w_proj)
 
+    t0 = time.perf_counter()
     run()
+    iters = max(2, min(8, int(budget_s / max(time.perf_counter() - t0, 1e-3))))
     times = []
     for _ in range(iters):
         t0 = time.perf_counter()
@@ -711,7 +714,7 @@ def main():
     if graph_ms is not None:
         out["ms_per_step_graph_replay"] = graph_ms
     if not args.no_cpu_baseline:
-        sample = args.cpu_sample_tokens or min(T, 8192)
+        sample = args.cpu_sample_tokens or min(T, 32768 if w.I <= 2048 else 8192)
         out["cpu_baseline"] = cpu_baseline(w, inputs, sample)
     print(json.dumps(out))
 
